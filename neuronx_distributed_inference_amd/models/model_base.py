@@ -89,6 +89,18 @@ class DecoderModel(nn.Module):
             config.hidden_size, config.vocab_size, bias=False, dtype=self.dtype,
             tp_degree=ec.tp_degree,
         )
+        self.kv_mgr = self.build_kv_manager(config)
+        self.sampler = (
+            Sampler(ec.on_device_sampling_config, config.vocab_size)
+            if ec.on_device_sampling_config
+            else None
+        )
+
+    # -- subclass hooks -------------------------------------------------
+    def build_kv_manager(self, config: InferenceConfig) -> nn.Module:
+        """Cache / state manager of this model. Subclasses with other cache
+        geometry (per-layer shapes, recurrent state) override this."""
+        ec = config.neuron_config
         head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
         n_kv_heads = getattr(config, "num_key_value_heads", config.num_attention_heads)
         # FP8 KV-cache quantization (ref kv_cache_manager.py:636-692): cache
@@ -108,7 +120,7 @@ class DecoderModel(nn.Module):
                 (ec.max_length + ec.pa_block_size - 1) // ec.pa_block_size
                 * ec.kv_cache_batch_size
             )
-            self.kv_mgr = BlockKVCacheManager(
+            return BlockKVCacheManager(
                 num_layers=self.num_layers, num_kv_heads=n_kv_heads,
                 head_dim=head_dim, num_blocks=num_blocks,
                 block_size=ec.pa_block_size, dtype=cache_dtype,
@@ -131,7 +143,7 @@ class DecoderModel(nn.Module):
                         ]
                     else:
                         layer_sizes = [sw] * self.num_layers
-            self.kv_mgr = KVCacheManager(
+            return KVCacheManager(
                 num_layers=self.num_layers,
                 num_kv_heads=n_kv_heads,
                 head_dim=head_dim,
@@ -142,13 +154,7 @@ class DecoderModel(nn.Module):
                 tp_degree=cache_tp,
                 layer_cache_sizes=layer_sizes,
             )
-        self.sampler = (
-            Sampler(ec.on_device_sampling_config, config.vocab_size)
-            if ec.on_device_sampling_config
-            else None
-        )
 
-    # -- subclass hooks -------------------------------------------------
     def build_rotary(self, config: InferenceConfig) -> RotaryEmbedding:
         head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
         return RotaryEmbedding(
@@ -160,6 +166,29 @@ class DecoderModel(nn.Module):
 
     def build_layers(self, config: InferenceConfig) -> nn.ModuleList:
         raise NotImplementedError
+
+    def begin_step(self, position_ids, seq_ids, block_table):
+        """Called once per forward before any layer; may install per-step
+        context on the cache manager and returns the block table to use."""
+        return block_table
+
+    def prepare_hidden(self, h: torch.Tensor) -> torch.Tensor:
+        """Embedding output -> residual stream (e.g. a widening cast)."""
+        return h
+
+    def layer_runs(self):
+        """Execution order as (layer index, callable) pairs. The default is
+        each layer once; models that repeat a span of layers with shared
+        weights return one entry per run."""
+        return list(enumerate(self.layers))
+
+    def before_layer_run(self, run_idx: int, h: torch.Tensor,
+                         h_embed: torch.Tensor) -> torch.Tensor:
+        return h
+
+    def finalize_logits(self, logits: torch.Tensor) -> torch.Tensor:
+        """Post-lm_head transform (e.g. a tanh soft cap)."""
+        return logits
 
     def build_norm(self, config: InferenceConfig) -> nn.Module:
         return RMSNorm(
@@ -187,6 +216,7 @@ class DecoderModel(nn.Module):
     ):
         phase = phase or self._phase(input_ids, position_ids)
         B, S = input_ids.shape
+        block_table = self.begin_step(position_ids, seq_ids, block_table)
         if block_table is not None and getattr(self.kv_mgr, "is_paged", False):
             from neuronx_distributed_inference_amd.modules.kvcache.block_kv_cache_manager import (
                 generate_slot_mapping,
@@ -219,8 +249,12 @@ class DecoderModel(nn.Module):
                 mask = (input_ids == tok).unsqueeze(-1)
                 h = h.masked_scatter(mask, feats.to(h.dtype).reshape(-1, h.shape[-1]))
         # models with non-1D rope (qwen2-vl m-rope) install a custom hook
-        cos_sin_fn = getattr(self, "_cos_sin_fn", None) or self.rotary.get_cos_sin
-        cos, sin = cos_sin_fn(position_ids, device=h.device)
+        if self.rotary is None and getattr(self, "_cos_sin_fn", None) is None:
+            cos = sin = None                 # position-free / bias-based models
+        else:
+            cos_sin_fn = getattr(self, "_cos_sin_fn", None) or self.rotary.get_cos_sin
+            cos, sin = cos_sin_fn(position_ids, device=h.device)
+        h = self.prepare_hidden(h)
         # int32 once here: the KV/attention kernels take int32 and a per-layer
         # .to() would launch 4 conversion kernels per layer per step
         position_ids = position_ids.to(torch.int32)
@@ -228,7 +262,9 @@ class DecoderModel(nn.Module):
             seq_ids = seq_ids.to(torch.int32)
         residual = None
         post_fns = getattr(self, "_layer_post_fns", None)
-        for li, layer in enumerate(self.layers):
+        h_embed = h
+        for ri, (li, layer) in enumerate(self.layer_runs()):
+            h = self.before_layer_run(ri, h, h_embed)
             if sp_active:
                 h, residual = layer(
                     h, residual, cos, sin, self.kv_mgr, position_ids, phase,
@@ -297,7 +333,7 @@ class DecoderModel(nn.Module):
         # (B, S, H) alive on every CTE
         if getattr(self, "eagle_capture_hidden", False):
             self.full_hidden = h
-        logits_shard = self.lm_head(h_last)  # (B, 1|S, V/tp)
+        logits_shard = self.finalize_logits(self.lm_head(h_last))  # (B, 1|S, V/tp)
 
         # rejection-sampling speculation reads the per-position top-Kg
         # distribution of every draft/verify pass (ref draft_probs /

@@ -106,7 +106,8 @@ class ModelWrapper:
         )
 
         device = next(self.model.parameters()).device
-        self.model.rotary.ensure_table(self.ec.max_length, device)
+        if self.model.rotary is not None:
+            self.model.rotary.ensure_table(self.ec.max_length, device)
         self._graphs = BucketedGraphModel()
 
         def fn(input_ids, position_ids, seq_ids, sampling_params):

@@ -29,7 +29,15 @@ class BlockKVCacheManager(nn.Module):
         block_size: int = 128,
         dtype: torch.dtype = torch.bfloat16,
         tp_degree: Optional[int] = None,
+        layer_kv_shapes: Optional[List[Tuple[int, int, int]]] = None,
+        state_slots: int = 0,
     ):
+        """`layer_kv_shapes`: optional per-layer (kv_heads, k_head_dim,
+        v_head_dim) for models whose layers differ or whose keys and values
+        have different head sizes; overrides num_kv_heads/head_dim.
+        `state_slots` > 0 attaches a :class:`RecurrentStateManager` as
+        ``self.state`` for models that also carry fixed-size per-sequence
+        state (linear recurrences, short-convolution tails)."""
         super().__init__()
         tp = tp_degree or ps.get_tensor_model_parallel_size()
         self.num_kv_heads_per_rank = max(num_kv_heads // tp, 1)
@@ -38,15 +46,25 @@ class BlockKVCacheManager(nn.Module):
         self.block_size = block_size
         self.num_layers = num_layers
         self.dtype = dtype
-        shape = (num_blocks, block_size, self.num_kv_heads_per_rank, head_dim)
+        if layer_kv_shapes is None:
+            layer_kv_shapes = [(num_kv_heads, head_dim, head_dim)] * num_layers
+        assert len(layer_kv_shapes) == num_layers
+        self.layer_kv_shapes = [(max(g // tp, 1), dk, dv) for g, dk, dv in layer_kv_shapes]
         self.k_caches = nn.ParameterList(
-            nn.Parameter(torch.zeros(shape, dtype=dtype), requires_grad=False)
-            for _ in range(num_layers)
+            nn.Parameter(torch.zeros((num_blocks, block_size, g, dk), dtype=dtype),
+                         requires_grad=False)
+            for g, dk, _ in self.layer_kv_shapes
         )
         self.v_caches = nn.ParameterList(
-            nn.Parameter(torch.zeros(shape, dtype=dtype), requires_grad=False)
-            for _ in range(num_layers)
+            nn.Parameter(torch.zeros((num_blocks, block_size, g, dv), dtype=dtype),
+                         requires_grad=False)
+            for g, _, dv in self.layer_kv_shapes
         )
+        self.state = RecurrentStateManager(state_slots) if state_slots > 0 else None
+
+    @property
+    def has_recurrent_state(self) -> bool:
+        return self.state is not None
 
     def estimate_bytes(self) -> int:
         return sum(k.numel() * k.element_size() * 2 for k in self.k_caches)
@@ -59,6 +77,10 @@ class BlockKVCacheManager(nn.Module):
     @property
     def block_table(self):
         return self._block_table
+
+    @property
+    def slot_mapping(self):
+        return self._slot_mapping
 
     def get_cache(self, layer_idx: int, bucket_len=None):
         return self.k_caches[layer_idx], self.v_caches[layer_idx]
@@ -94,6 +116,39 @@ class BlockKVCacheManager(nn.Module):
             k.data.zero_()
         for v in self.v_caches:
             v.data.zero_()
+        if self.state is not None:
+            self.state.reset()
+
+
+class RecurrentStateManager(nn.Module):
+    """Fixed-size per-sequence state beside the KV cache: one fp32 tensor
+    (slots, *shape) per registered key. A slot is the engine's seq_id, the
+    same index that selects a linear-cache row; kernels start from zeros
+    when a row's first token has position 0, so a slot that is handed to a
+    new request needs no clearing."""
+
+    def __init__(self, num_slots: int):
+        super().__init__()
+        self.num_slots = num_slots
+        self.tensors = nn.ParameterDict()
+
+    @staticmethod
+    def _key(name: str) -> str:
+        return name.replace(".", "_")
+
+    def register(self, name: str, shape, dtype: torch.dtype = torch.float32):
+        self.tensors[self._key(name)] = nn.Parameter(
+            torch.zeros((self.num_slots, *shape), dtype=dtype), requires_grad=False)
+
+    def get(self, name: str) -> torch.Tensor:
+        return self.tensors[self._key(name)].data
+
+    def estimate_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.tensors.values())
+
+    def reset(self):
+        for t in self.tensors.values():
+            t.data.zero_()
 
 
 def generate_slot_mapping(block_table: torch.Tensor, positions: torch.Tensor,

@@ -1,0 +1,70 @@
+"""Gated delta-rule token mixer core (a linear recurrence with matrix state).
+
+Per head the state is a (dim x vdim) fp32 matrix ``M`` updated once per token
+
+    M <- diag(d_t) M            d_t = exp(-exp(A_log) * softplus(a_t + dt_bias))
+    u  = beta_t (v_t - M^T k_t)                  (delta-rule correction)
+    M <- M + k_t u^T
+    o_t = M^T q_t                                (reads the fresh write)
+
+with one decay per head AND key channel, unit-norm q/k (q also scaled by
+dim^-1/2), beta a sigmoid. q/k/v first pass a short causal convolution and
+SiLU; the output is RMS-normalised per head, scaled by a weight shared
+across heads and multiplied by a sigmoid gate. ``a_t`` and the gate come
+through low-rank two-stage projections whose second stages live here.
+
+State (``M`` and the convolution tail) is engine state in the cache
+manager's :class:`RecurrentStateManager`, keyed by this module's name and
+the layer run, so prompts can be cut anywhere and decode continues from
+prefill. The first-stage projections of the layer input are the caller's.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from neuronx_distributed_inference_amd.modules.conv import CausalShortConv
+from neuronx_distributed_inference_amd.ops import seqmix
+from neuronx_distributed_inference_amd.parallel.layers import ColumnParallelLinear
+
+
+class GatedDeltaRule(nn.Module):
+    def __init__(self, num_heads: int, num_kv_heads: int, dim: int, vdim: int,
+                 conv_taps: int, decay_rank: int, gate_rank: int, eps: float,
+                 dtype: torch.dtype, tp_degree: int = 1):
+        super().__init__()
+        assert num_heads % num_kv_heads == 0
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.dim = dim
+        self.vdim = vdim
+        self.eps = float(eps)
+        self.qkv_channels = 2 * num_kv_heads * dim + num_heads * vdim
+        self.conv = CausalShortConv(self.qkv_channels, conv_taps, activation="silu")
+        self.a2 = ColumnParallelLinear(decay_rank, num_heads * dim, dtype=dtype,
+                                       tp_degree=tp_degree)
+        self.g2 = ColumnParallelLinear(gate_rank, num_heads * vdim, dtype=dtype,
+                                       tp_degree=tp_degree)
+        f32 = dict(dtype=torch.float32)
+        self.A_log = nn.Parameter(torch.zeros(num_heads, **f32), requires_grad=False)
+        self.dt_bias = nn.Parameter(torch.zeros(num_heads * dim, **f32), requires_grad=False)
+        self.norm_weight = nn.Parameter(torch.ones(vdim, **f32), requires_grad=False)
+
+    def state_shapes(self):
+        return {"conv": self.conv.state_shape(),
+                "mem": (self.num_heads, self.dim, self.vdim)}
+
+    def forward(self, qkv: torch.Tensor, beta: torch.Tensor, a_low: torch.Tensor,
+                g_low: torch.Tensor, states, key: str,
+                step: seqmix.StepLayout) -> torch.Tensor:
+        """qkv (B,S,q|k|v channels) raw projections, beta (B,S,H) logits,
+        a_low / g_low the first-stage low-rank projections. `states` is the
+        RecurrentStateManager, `key` this layer run's prefix in it."""
+        qkv_c = self.conv(qkv, states.get(key + ".conv"), step, out_dtype=torch.float32)
+        a = self.a2(a_low)
+        gate = self.g2(g_low)
+        return seqmix.gated_delta_rule(
+            qkv_c, beta, a, self.dt_bias, self.A_log, gate, self.norm_weight,
+            self.eps, states.get(key + ".mem"), step, self.num_kv_heads, self.dim,
+            self.vdim, out_dtype=a.dtype)

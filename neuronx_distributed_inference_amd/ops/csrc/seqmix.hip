@@ -1,0 +1,564 @@
+// Sequence-mixing kernels for hybrid models (gfx950): bias-free LayerNorm on
+// an fp32 residual stream, short causal convolutions with a carried tail,
+// paged KV scatter with distinct K/V head sizes, windowed softmax attention
+// with a log-distance penalty and always-visible first tokens, and the gated
+// delta-rule linear recurrence.
+//
+// Built as a plain C-ABI shared library (no torch headers): the Python side
+// passes raw device pointers and the current HIP stream, so the kernels are
+// stream-ordered with the surrounding torch ops and hipGraph-capturable.
+//
+// Step layout shared by all kernels: activations are (B, S, ...) row-major;
+// `pos` (B,S) int32 holds each token's position or -1 for padding; the real
+// tokens of a row sit at columns 0..n-1 with consecutive positions; `seq`
+// (B) int32 is the row's state slot or -1; `nvalid` (B) int32 is n.
+// Statistics, scores, softmax, decays and the recurrent state are fp32
+// regardless of the activation type.
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#define WAVE 64
+#define DEV __device__ __forceinline__
+
+typedef __hip_bfloat16 bf16;
+
+template <typename T> DEV float ldf(const T* p);
+template <> DEV float ldf<float>(const float* p) { return *p; }
+template <> DEV float ldf<bf16>(const bf16* p) { return __bfloat162float(*p); }
+template <typename T> DEV void stf(T* p, float v);
+template <> DEV void stf<float>(float* p, float v) { *p = v; }
+template <> DEV void stf<bf16>(bf16* p, float v) { *p = __float2bfloat16(v); }
+
+DEV float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+DEV float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+DEV float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
+DEV float softplusf_(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// ---------------------------------------------------------------- LayerNorm
+// one wave per row; mean, then variance of the deviations (both fp32)
+template <typename TOut>
+__global__ void layer_norm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                  TOut* __restrict__ out, long rows, int C, float eps) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const long row = (long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (row >= rows) return;
+    const float* xr = x + row * C;
+    float s = 0.f;
+    for (int c = lane; c < C; c += WAVE) s += xr[c];
+    const float mean = wave_sum(s) / C;
+    float v = 0.f;
+    for (int c = lane; c < C; c += WAVE) { float d = xr[c] - mean; v += d * d; }
+    const float inv = 1.f / sqrtf(wave_sum(v) / C + eps);
+    TOut* o = out + row * C;
+    for (int c = lane; c < C; c += WAVE) stf<TOut>(o + c, (xr[c] - mean) * inv * w[c]);
+}
+
+// ------------------------------------------------------------- short conv
+// y[b,t,c] = act(sum_j w[c,j] * x[b, t-R+j, c]) (+ x[b,t,c]); columns before
+// the step come from the carried tail (oldest first), positions < 0 are zero
+template <typename TIn, typename TOut>
+__global__ void short_conv_kernel(const TIn* __restrict__ x, const float* __restrict__ w,
+                                  const float* __restrict__ tail, const int* __restrict__ pos,
+                                  const int* __restrict__ seq, TOut* __restrict__ y,
+                                  int B, int S, int C, int taps, int act_silu, int residual) {
+    const long total = (long)B * S * C;
+    const int R = taps - 1;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int c = idx % C;
+        const long bt = idx / C;
+        const int t = bt % S;
+        const int b = bt / S;
+        const int p = pos[bt];
+        const int slot = seq[b];
+        if (p < 0 || slot < 0) { stf<TOut>(y + idx, 0.f); continue; }
+        const float* wr = w + (long)c * taps;
+        float acc = 0.f;
+        for (int j = 0; j < taps; ++j) {
+            const int col = t - R + j;
+            float xv;
+            if (col >= 0) {
+                xv = ldf<TIn>(x + ((long)b * S + col) * C + c);
+            } else {
+                const int ps = p - R + j;              // source position
+                xv = ps < 0 ? 0.f : tail[((long)slot * R + (R + col)) * C + c];
+            }
+            acc += wr[j] * xv;
+        }
+        if (act_silu) acc = acc * sigmoidf_(acc);
+        if (residual) acc += ldf<TIn>(x + idx);
+        stf<TOut>(y + idx, acc);
+    }
+}
+
+// new tail = last R inputs of (old tail ++ this step's inputs); one thread per
+// (row, channel) so the in-place shift is private to the thread
+template <typename TIn>
+__global__ void short_conv_commit_kernel(const TIn* __restrict__ x, float* __restrict__ tail,
+                                         const int* __restrict__ pos, const int* __restrict__ seq,
+                                         const int* __restrict__ nvalid, int B, int S, int C, int R) {
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long)B * C) return;
+    const int c = idx % C;
+    const int b = idx / C;
+    const int slot = seq[b];
+    const int n = nvalid[b];
+    if (slot < 0 || n <= 0) return;
+    const int p0 = pos[(long)b * S];
+    float* tr = tail + (long)slot * R * C + c;
+    for (int r = 0; r < R; ++r) {
+        const int col = n - R + r;
+        float v;
+        if (col >= 0) v = ldf<TIn>(x + ((long)b * S + col) * C + c);
+        else v = (p0 + col) < 0 ? 0.f : tr[(long)(R + col) * C];
+        tr[(long)r * C] = v;
+    }
+}
+
+// ------------------------------------------------------------ paged KV write
+template <typename T>
+__global__ void paged_kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc,
+                                      const T* __restrict__ k, long kstride,
+                                      const T* __restrict__ v, long vstride,
+                                      const int* __restrict__ slots, long N, int GDk, int GDv,
+                                      long nslots) {
+    const int per = GDk + GDv;
+    const long total = N * per;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const long tok = idx / per;
+        const int e = idx % per;
+        const int s = slots[tok];
+        if (s < 0 || s >= nslots) continue;
+        if (e < GDk) kc[(long)s * GDk + e] = k[tok * kstride + e];
+        else vc[(long)s * GDv + (e - GDk)] = v[tok * vstride + (e - GDk)];
+    }
+}
+
+// ------------------------------------------------- windowed biased attention
+// One wave per (token, query head). Visible keys of query position i:
+// j in [0, min(keep, lo)) and j in [lo, i], lo = max(0, i-window+1). Lanes
+// take one key each for the scores (online softmax over 64-key tiles), then
+// one value channel each for P.V.
+#define ATT_WAVES 4
+#define ATT_MAXR 4   // value head size <= 64*ATT_MAXR
+
+template <typename T, typename TOut>
+__global__ void __launch_bounds__(ATT_WAVES * WAVE)
+window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ kc,
+                   const T* __restrict__ vc, const int* __restrict__ pos,
+                   const int* __restrict__ btab, int max_blocks, const float* __restrict__ r1,
+                   const float* __restrict__ r2, const T* __restrict__ gate, long gstride,
+                   TOut* __restrict__ out, long ntok, int H, int G, int Dk, int Dv,
+                   int bsz, int S, float scale, int window, int keep) {
+    extern __shared__ float qs[];                      // ATT_WAVES * Dk
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wv = threadIdx.x / WAVE;
+    const long wid = (long)blockIdx.x * ATT_WAVES + wv;
+    const bool live = wid < ntok * H;
+    const long tok = live ? wid / H : 0;
+    const int h = live ? (int)(wid % H) : 0;
+    const int i = live ? pos[tok] : -1;
+    float* myq = qs + wv * Dk;
+    if (i >= 0) {
+        const T* qp = q + tok * qstride + (long)h * Dk;
+        for (int d = lane; d < Dk; d += WAVE) myq[d] = ldf<T>(qp + d) * scale;
+    }
+    __syncthreads();
+    if (i < 0) return;
+    const int b = tok / S;
+    const int g = h / (H / G);
+    const int* bt = btab + (long)b * max_blocks;
+    const int lo = max(0, i - window + 1);
+    const int nfirst = min(keep, lo);
+    const int n = nfirst + (i - lo + 1);
+    const float a1 = r1[h], a2 = r2[h];
+    float m_run = -INFINITY, l_run = 0.f;
+    float acc[ATT_MAXR];
+#pragma unroll
+    for (int r = 0; r < ATT_MAXR; ++r) acc[r] = 0.f;
+    const long krow = (long)G * Dk, vrow = (long)G * Dv;
+
+    for (int base = 0; base < n; base += WAVE) {
+        const int m = base + lane;
+        float s = -INFINITY;
+        long slot = 0;
+        if (m < n) {
+            const int j = m < nfirst ? m : lo + (m - nfirst);
+            slot = (long)bt[j / bsz] * bsz + (j % bsz);
+            const T* kp = kc + slot * krow + (long)g * Dk;
+            float dot = 0.f;
+            if constexpr (sizeof(T) == 2) {
+                if ((Dk & 7) == 0) {
+                    for (int d = 0; d < Dk; d += 8) {
+                        const uint4 raw = *reinterpret_cast<const uint4*>(kp + d);
+                        const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            dot += __uint_as_float(u[e] << 16) * myq[d + 2 * e];
+                            dot += __uint_as_float(u[e] & 0xffff0000u) * myq[d + 2 * e + 1];
+                        }
+                    }
+                } else {
+                    for (int d = 0; d < Dk; ++d) dot += ldf<T>(kp + d) * myq[d];
+                }
+            } else {
+                if ((Dk & 3) == 0) {
+                    for (int d = 0; d < Dk; d += 4) {
+                        const float4 kv = *reinterpret_cast<const float4*>(kp + d);
+                        dot += kv.x * myq[d] + kv.y * myq[d + 1] + kv.z * myq[d + 2] +
+                               kv.w * myq[d + 3];
+                    }
+                } else {
+                    for (int d = 0; d < Dk; ++d) dot += ldf<T>(kp + d) * myq[d];
+                }
+            }
+            s = dot - a1 * log1pf(a2 * (float)(i - j));
+        }
+        const float m_new = fmaxf(m_run, wave_max(s));
+        const float p = (m < n) ? expf(s - m_new) : 0.f;
+        const float corr = expf(m_run - m_new);        // 0 on the first tile
+        l_run = l_run * corr + wave_sum(p);
+        m_run = m_new;
+#pragma unroll
+        for (int r = 0; r < ATT_MAXR; ++r) acc[r] *= corr;
+        const int cnt = min(WAVE, n - base);
+        for (int mm = 0; mm < cnt; ++mm) {
+            const float pj = __shfl(p, mm, WAVE);
+            const long sj = __shfl((int)slot, mm, WAVE);
+            const T* vp = vc + sj * vrow + (long)g * Dv;
+#pragma unroll
+            for (int r = 0; r < ATT_MAXR; ++r) {
+                const int d = lane + r * WAVE;
+                if (d < Dv) acc[r] += pj * ldf<T>(vp + d);
+            }
+        }
+    }
+    const float inv = 1.f / l_run;
+    TOut* op = out + (tok * H + h) * (long)Dv;
+    const T* gp = gate ? gate + tok * gstride + (long)h * Dv : nullptr;
+#pragma unroll
+    for (int r = 0; r < ATT_MAXR; ++r) {
+        const int d = lane + r * WAVE;
+        if (d < Dv) {
+            float o = acc[r] * inv;
+            if (gp) o *= sigmoidf_(ldf<T>(gp + d));
+            stf<TOut>(op + d, o);
+        }
+    }
+}
+
+// ------------------------------------------------------- gated delta rule
+// One workgroup per (row, head); thread j owns column j of the (D x Dv) state
+// in registers, so the recurrence needs no cross-thread traffic. Tokens are
+// processed in chunks of GD_TC: a parallel phase prepares unit q/k, decays,
+// beta in LDS; a serial phase runs the recurrence; a parallel phase applies
+// the per-head RMS norm and the sigmoid gate.
+#define GD_TC 8
+
+#define GD_MAXTHR 256
+
+template <int DK, typename T, typename TOut>
+__global__ void __launch_bounds__(GD_MAXTHR)
+gated_delta_kernel(const float* __restrict__ qkv, long cstride,
+                                   const T* __restrict__ beta, long bstride,
+                                   const T* __restrict__ a, long astride,
+                                   const T* __restrict__ gate, long gstride,
+                                   const float* __restrict__ dt_bias,
+                                   const float* __restrict__ a_log,
+                                   const float* __restrict__ norm_w, float eps,
+                                   float* __restrict__ state, const int* __restrict__ pos,
+                                   const int* __restrict__ seq, const int* __restrict__ nvalid,
+                                   TOut* __restrict__ out, int S, int H, int G, int D, int Dv) {
+    extern __shared__ float lds[];
+    const int nthr = blockDim.x;
+    const int Dvp = nthr;
+    float* qs = lds;                         // GD_TC * DK
+    float* ks = qs + GD_TC * DK;
+    float* gs = ks + GD_TC * DK;
+    float* os = gs + GD_TC * DK;             // GD_TC * Dvp
+    float* bs = os + GD_TC * Dvp;            // GD_TC
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int slot = seq[b];
+    const int n = nvalid[b];
+    if (slot < 0 || n <= 0) return;          // uniform over the workgroup
+    const int j = threadIdx.x;
+    const int lane = j & (WAVE - 1), wv = j / WAVE, nw = nthr / WAVE;
+    const bool act = j < Dv;
+    const int g = h / (H / G);
+    const int p0 = pos[(long)b * S];
+    float* st = state + ((long)slot * H + h) * D * Dv;
+    float s[DK];
+#pragma unroll
+    for (int i = 0; i < DK; ++i)
+        s[i] = (act && i < D && p0 > 0) ? st[(long)i * Dv + j] : 0.f;
+    const float neg_rate = -expf(a_log[h]);
+    const float qscale = 1.f / sqrtf((float)D);
+
+    for (int t0 = 0; t0 < n; t0 += GD_TC) {
+        const int tc = min(GD_TC, n - t0);
+        const long row0 = (long)b * S + t0;
+        // ---- parallel: unit q / k
+        for (int r = wv; r < 2 * tc; r += nw) {
+            const int tk = r >> 1, which = r & 1;
+            const float* src = qkv + (row0 + tk) * cstride + (which ? G * D : 0) + g * D;
+            float ss = 0.f;
+            for (int i = lane; i < D; i += WAVE) { float x = src[i]; ss += x * x; }
+            float inv = 1.f / sqrtf(wave_sum(ss) + 1e-6f);
+            if (!which) inv *= qscale;
+            float* dst = (which ? ks : qs) + tk * DK;
+            for (int i = lane; i < DK; i += WAVE) dst[i] = i < D ? src[i] * inv : 0.f;
+        }
+        // ---- parallel: decays and beta
+        for (int idx = j; idx < tc * DK; idx += nthr) {
+            const int tk = idx / DK, i = idx % DK;
+            float dv = 1.f;
+            if (i < D) {
+                const float z = ldf<T>(a + (row0 + tk) * astride + h * D + i) + dt_bias[h * D + i];
+                dv = expf(neg_rate * softplusf_(z));
+            }
+            gs[idx] = dv;
+        }
+        if (j < tc) bs[j] = sigmoidf_(ldf<T>(beta + (row0 + j) * bstride + h));
+        float vreg[GD_TC], oreg[GD_TC];
+#pragma unroll
+        for (int tk = 0; tk < GD_TC; ++tk)
+            vreg[tk] = (act && tk < tc)
+                ? qkv[(row0 + tk) * cstride + 2 * G * D + (long)h * Dv + j] : 0.f;
+        __syncthreads();
+        // ---- serial recurrence over the chunk
+#pragma unroll
+        for (int tk = 0; tk < GD_TC; ++tk) {
+            oreg[tk] = 0.f;
+            if (tk < tc) {
+                const float4* g4 = reinterpret_cast<const float4*>(gs + tk * DK);
+                const float4* k4 = reinterpret_cast<const float4*>(ks + tk * DK);
+                const float4* q4 = reinterpret_cast<const float4*>(qs + tk * DK);
+                float dot = 0.f;
+#pragma unroll
+                for (int i = 0; i < DK / 4; ++i) {
+                    const float4 gg = g4[i], kk = k4[i];
+                    s[4 * i] *= gg.x; dot += s[4 * i] * kk.x;
+                    s[4 * i + 1] *= gg.y; dot += s[4 * i + 1] * kk.y;
+                    s[4 * i + 2] *= gg.z; dot += s[4 * i + 2] * kk.z;
+                    s[4 * i + 3] *= gg.w; dot += s[4 * i + 3] * kk.w;
+                }
+                const float u = bs[tk] * (vreg[tk] - dot);
+                float o = 0.f;
+#pragma unroll
+                for (int i = 0; i < DK / 4; ++i) {
+                    const float4 kk = k4[i], qq = q4[i];
+                    s[4 * i] += kk.x * u; o += s[4 * i] * qq.x;
+                    s[4 * i + 1] += kk.y * u; o += s[4 * i + 1] * qq.y;
+                    s[4 * i + 2] += kk.z * u; o += s[4 * i + 2] * qq.z;
+                    s[4 * i + 3] += kk.w * u; o += s[4 * i + 3] * qq.w;
+                }
+                oreg[tk] = o;
+            }
+        }
+#pragma unroll
+        for (int tk = 0; tk < GD_TC; ++tk) os[tk * Dvp + j] = act ? oreg[tk] : 0.f;
+        __syncthreads();
+        // ---- parallel: RMS norm over the value channels, weight, gate
+        for (int tk = wv; tk < tc; tk += nw) {
+            float ss = 0.f;
+            for (int c = lane; c < Dv; c += WAVE) { float o = os[tk * Dvp + c]; ss += o * o; }
+            const float inv = 1.f / sqrtf(wave_sum(ss) / Dv + eps);
+            const T* gp = gate + (row0 + tk) * gstride + (long)h * Dv;
+            TOut* op = out + ((row0 + tk) * H + h) * (long)Dv;
+            for (int c = lane; c < Dv; c += WAVE)
+                stf<TOut>(op + c, os[tk * Dvp + c] * inv * norm_w[c] * sigmoidf_(ldf<T>(gp + c)));
+        }
+        __syncthreads();
+    }
+    if (act) {
+#pragma unroll
+        for (int i = 0; i < DK; ++i)
+            if (i < D) st[(long)i * Dv + j] = s[i];
+    }
+}
+
+// ------------------------------------------------------------- elementwise
+template <typename T>
+__global__ void softcap_kernel(const T* __restrict__ in, float* __restrict__ out, long n,
+                               float cap) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (long)gridDim.x * blockDim.x)
+        out[i] = cap * tanhf(ldf<T>(in + i) / cap);
+}
+
+// x += sa*a (+ sb*b), fp32 residual stream
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ a, float sa,
+                                    const T* __restrict__ b, float sb, long n) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (long)gridDim.x * blockDim.x) {
+        float v = x[i] + sa * ldf<T>(a + i);
+        if (b) v += sb * ldf<T>(b + i);
+        x[i] = v;
+    }
+}
+
+// out[r, c] = gelu_tanh(gu[r, c]) * gu[r, I + c]
+template <typename T>
+__global__ void gelu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, long rows, int I) {
+    const long total = rows * I;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / I;
+        const int c = idx % I;
+        const float z = ldf<T>(gu + r * 2 * I + c);
+        const float u = ldf<T>(gu + r * 2 * I + I + c);
+        const float ge = 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+        stf<T>(out + idx, ge * u);
+    }
+}
+
+// =================================================================== C ABI
+static inline int grid_for(long total, int block, int cap = 8192) {
+    long g = (total + block - 1) / block;
+    if (g < 1) g = 1;
+    return (int)(g > cap ? cap : g);
+}
+
+extern "C" {
+
+int nx_layer_norm(const float* x, const float* w, void* out, int out_bf16, long rows, int C,
+                  float eps, hipStream_t st) {
+    if (rows <= 0) return 0;
+    const int wpb = 4;
+    dim3 grid((unsigned)((rows + wpb - 1) / wpb)), block(wpb * WAVE);
+    if (out_bf16) layer_norm_kernel<bf16><<<grid, block, 0, st>>>(x, w, (bf16*)out, rows, C, eps);
+    else layer_norm_kernel<float><<<grid, block, 0, st>>>(x, w, (float*)out, rows, C, eps);
+    return (int)hipGetLastError();
+}
+
+int nx_short_conv(const void* x, int x_bf16, const float* w, const float* tail, const int* pos,
+                  const int* seq, void* y, int y_bf16, int B, int S, int C, int taps,
+                  int act_silu, int residual, hipStream_t st) {
+    const long total = (long)B * S * C;
+    if (total <= 0) return 0;
+    dim3 grid(grid_for(total, 256)), block(256);
+#define SC(TI, TO) short_conv_kernel<TI, TO><<<grid, block, 0, st>>>( \
+        (const TI*)x, w, tail, pos, seq, (TO*)y, B, S, C, taps, act_silu, residual)
+    if (x_bf16 && y_bf16) SC(bf16, bf16);
+    else if (x_bf16) SC(bf16, float);
+    else if (y_bf16) SC(float, bf16);
+    else SC(float, float);
+#undef SC
+    return (int)hipGetLastError();
+}
+
+int nx_short_conv_commit(const void* x, int x_bf16, float* tail, const int* pos, const int* seq,
+                         const int* nvalid, int B, int S, int C, int R, hipStream_t st) {
+    const long total = (long)B * C;
+    if (total <= 0 || R <= 0) return 0;
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (x_bf16) short_conv_commit_kernel<bf16><<<grid, block, 0, st>>>(
+        (const bf16*)x, tail, pos, seq, nvalid, B, S, C, R);
+    else short_conv_commit_kernel<float><<<grid, block, 0, st>>>(
+        (const float*)x, tail, pos, seq, nvalid, B, S, C, R);
+    return (int)hipGetLastError();
+}
+
+int nx_paged_kv_write(void* kc, void* vc, const void* k, long kstride, const void* v,
+                      long vstride, int is_bf16, const int* slots, long N, int GDk, int GDv,
+                      long nslots, hipStream_t st) {
+    const long total = N * (GDk + GDv);
+    if (total <= 0) return 0;
+    dim3 grid(grid_for(total, 256)), block(256);
+    if (is_bf16) paged_kv_write_kernel<bf16><<<grid, block, 0, st>>>(
+        (bf16*)kc, (bf16*)vc, (const bf16*)k, kstride, (const bf16*)v, vstride, slots, N, GDk,
+        GDv, nslots);
+    else paged_kv_write_kernel<float><<<grid, block, 0, st>>>(
+        (float*)kc, (float*)vc, (const float*)k, kstride, (const float*)v, vstride, slots, N,
+        GDk, GDv, nslots);
+    return (int)hipGetLastError();
+}
+
+int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, const int* pos,
+                   const int* btab, int max_blocks, const float* r1, const float* r2,
+                   const void* gate, long gstride, void* out, int io_bf16, int out_bf16,
+                   int B, int S, int H, int G, int Dk, int Dv, int bsz, float scale, int window,
+                   int keep, hipStream_t st) {
+    const long ntok = (long)B * S;
+    if (ntok <= 0) return 0;
+    if (Dv > WAVE * ATT_MAXR || H % G != 0) return -1;
+    const long waves = ntok * H;
+    dim3 grid((unsigned)((waves + ATT_WAVES - 1) / ATT_WAVES)), block(ATT_WAVES * WAVE);
+    const size_t sh = (size_t)ATT_WAVES * Dk * sizeof(float);
+#define WA(T, TO) window_attn_kernel<T, TO><<<grid, block, sh, st>>>( \
+        (const T*)q, qstride, (const T*)kc, (const T*)vc, pos, btab, max_blocks, r1, r2, \
+        (const T*)gate, gstride, (TO*)out, ntok, H, G, Dk, Dv, bsz, S, scale, window, keep)
+    if (io_bf16 && out_bf16) WA(bf16, bf16);
+    else if (io_bf16) WA(bf16, float);
+    else if (out_bf16) return -2;
+    else WA(float, float);
+#undef WA
+    return (int)hipGetLastError();
+}
+
+int nx_gated_delta(const float* qkv, long cstride, const void* beta, long bstride, const void* a,
+                   long astride, const void* gate, long gstride, const float* dt_bias,
+                   const float* a_log, const float* norm_w, float eps, float* state,
+                   const int* pos, const int* seq, const int* nvalid, void* out, int in_bf16,
+                   int B, int S, int H, int G, int D, int Dv, hipStream_t st) {
+    if (B <= 0 || S <= 0) return 0;
+    if (D > 256 || Dv > GD_MAXTHR || H % G != 0) return -1;
+    const int nthr = ((Dv + WAVE - 1) / WAVE) * WAVE;
+    const int DK = D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
+    const size_t sh = (size_t)(3 * GD_TC * DK + GD_TC * nthr + GD_TC) * sizeof(float);
+    dim3 grid(H, B), block(nthr);
+#define GD(DKV, T) gated_delta_kernel<DKV, T, T><<<grid, block, sh, st>>>( \
+        qkv, cstride, (const T*)beta, bstride, (const T*)a, astride, (const T*)gate, gstride, \
+        dt_bias, a_log, norm_w, eps, state, pos, seq, nvalid, (T*)out, S, H, G, D, Dv)
+#define GDT(DKV) do { if (in_bf16) GD(DKV, bf16); else GD(DKV, float); } while (0)
+    switch (DK) {
+        case 32: GDT(32); break;
+        case 64: GDT(64); break;
+        case 128: GDT(128); break;
+        default: GDT(256); break;
+    }
+#undef GDT
+#undef GD
+    return (int)hipGetLastError();
+}
+
+int nx_softcap(const void* in, int in_bf16, float* out, long n, float cap, hipStream_t st) {
+    if (n <= 0) return 0;
+    dim3 grid(grid_for(n, 256)), block(256);
+    if (in_bf16) softcap_kernel<bf16><<<grid, block, 0, st>>>((const bf16*)in, out, n, cap);
+    else softcap_kernel<float><<<grid, block, 0, st>>>((const float*)in, out, n, cap);
+    return (int)hipGetLastError();
+}
+
+int nx_residual_add(float* x, const void* a, float sa, const void* b, float sb, int is_bf16,
+                    long n, hipStream_t st) {
+    if (n <= 0) return 0;
+    dim3 grid(grid_for(n, 256)), block(256);
+    if (is_bf16) residual_add_kernel<bf16><<<grid, block, 0, st>>>(
+        x, (const bf16*)a, sa, (const bf16*)b, sb, n);
+    else residual_add_kernel<float><<<grid, block, 0, st>>>(
+        x, (const float*)a, sa, (const float*)b, sb, n);
+    return (int)hipGetLastError();
+}
+
+int nx_gelu_mul(const void* gu, void* out, int is_bf16, long rows, int I, hipStream_t st) {
+    if (rows <= 0) return 0;
+    dim3 grid(grid_for(rows * I, 256)), block(256);
+    if (is_bf16) gelu_mul_kernel<bf16><<<grid, block, 0, st>>>((const bf16*)gu, (bf16*)out, rows, I);
+    else gelu_mul_kernel<float><<<grid, block, 0, st>>>((const float*)gu, (float*)out, rows, I);
+    return (int)hipGetLastError();
+}
+
+}  // extern "C"

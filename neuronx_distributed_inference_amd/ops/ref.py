@@ -209,3 +209,171 @@ def topk_topp_sample(
         j = min(j, k - 1)
         out[b] = idxs[b, j]
     return out
+
+
+# ----------------------------------------------------------------------
+# Sequence-mixing ops of the hybrid (windowed attention + linear
+# recurrence) models. All take the engine's ragged step layout: (B, S)
+# rows whose real tokens sit at columns 0..n-1 with consecutive positions
+# p0..p0+n-1; pad columns carry position -1 and pad rows seq_id -1.
+
+def layer_norm(x: torch.Tensor, weight: torch.Tensor, eps: float,
+               out_dtype: torch.dtype) -> torch.Tensor:
+    """Bias-free LayerNorm with fp32 statistics."""
+    xf = x.float()
+    mu = xf.mean(-1, keepdim=True)
+    xc = xf - mu
+    var = (xc * xc).mean(-1, keepdim=True)
+    return (xc * torch.rsqrt(var + eps) * weight.float()).to(out_dtype)
+
+
+def _row_extent(positions: torch.Tensor):
+    valid = positions >= 0
+    return valid.sum(-1), positions[:, 0]
+
+
+def _masked_tail(tail_row: torch.Tensor, p0: int) -> torch.Tensor:
+    """Tail rows hold inputs p0-R..p0-1 (oldest first); the ones that lie
+    before the sequence start read as zero."""
+    R = tail_row.shape[0]
+    src = p0 - R + torch.arange(R, device=tail_row.device)
+    return tail_row * (src >= 0).view(R, 1).to(tail_row.dtype)
+
+
+def short_conv(x, w, tail, positions, seq_ids, activation="none",
+               residual=False, out_dtype=torch.float32):
+    """Depthwise causal convolution over time with a carried tail:
+    y_t = sum_j w[:, j] * x_{t-(taps-1)+j}; the last column of `w`
+    multiplies the current token. x (B,S,C); w (C,taps); tail
+    (slots, taps-1, C) fp32."""
+    B, S, C = x.shape
+    taps = w.shape[1]
+    R = taps - 1
+    xf = x.float()
+    wf = w.float()
+    y = torch.zeros(B, S, C, dtype=torch.float32, device=x.device)
+    n_valid, p0s = _row_extent(positions)
+    for b in range(B):
+        slot = int(seq_ids[b])
+        n = int(n_valid[b])
+        if slot < 0 or n == 0:
+            continue
+        ext = torch.cat([_masked_tail(tail[slot].float(), int(p0s[b])), xf[b, :n]], 0)
+        acc = torch.zeros(n, C, dtype=torch.float32, device=x.device)
+        for j in range(taps):
+            acc = acc + wf[:, j] * ext[j:j + n]
+        y[b, :n] = acc
+    if activation == "silu":
+        y = torch.nn.functional.silu(y)
+    if residual:
+        y = y + xf
+    return y.to(out_dtype)
+
+
+def short_conv_commit(x, tail, positions, seq_ids):
+    """Advance the carried tail by this step's inputs."""
+    B = x.shape[0]
+    R = tail.shape[1]
+    n_valid, p0s = _row_extent(positions)
+    for b in range(B):
+        slot = int(seq_ids[b])
+        n = int(n_valid[b])
+        if slot < 0 or n == 0:
+            continue
+        ext = torch.cat([_masked_tail(tail[slot].float(), int(p0s[b])),
+                         x[b, :n].float()], 0)
+        tail[slot] = ext[-R:].to(tail.dtype)
+
+
+def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping):
+    """k_new (N,G,Dk), v_new (N,G,Dv) into (blocks, block, G, D*) caches;
+    K and V may have different head sizes."""
+    ok = slot_mapping >= 0
+    idx = slot_mapping[ok].long()
+    kc = k_cache.view(-1, *k_cache.shape[2:])
+    vc = v_cache.view(-1, *v_cache.shape[2:])
+    kc[idx] = k_new[ok].to(kc.dtype)
+    vc[idx] = v_new[ok].to(vc.dtype)
+
+
+def window_bias_attention(q, k_cache, v_cache, positions, block_table, r1, r2,
+                          scale, window, keep_first, gate=None,
+                          out_dtype=torch.float32):
+    """Softmax attention of ragged queries against a paged cache. Query at
+    position i sees key j <= i when i-j < window or j < keep_first; the
+    score is q.k*scale - r1_h*log1p(r2_h*(i-j)). q (B,S,H,Dk) ->
+    (B,S,H*Dv), optionally multiplied by sigmoid(gate)."""
+    B, S, H, Dk = q.shape
+    G, Dv = v_cache.shape[2], v_cache.shape[3]
+    bs = k_cache.shape[1]
+    L = int(positions.max()) + 1 if positions.numel() else 0
+    out = torch.zeros(B, S, H, Dv, dtype=torch.float32, device=q.device)
+    if L > 0:
+        nb = (L + bs - 1) // bs
+        bt = block_table[:, :nb].long().clamp(min=0)
+        k = k_cache[bt].reshape(B, nb * bs, G, Dk)[:, :L].float()
+        v = v_cache[bt].reshape(B, nb * bs, G, Dv)[:, :L].float()
+        rep = H // G
+        k = k.repeat_interleave(rep, dim=2)
+        v = v.repeat_interleave(rep, dim=2)
+        s = torch.einsum("bshd,blhd->bhsl", q.float(), k) * scale
+        i = positions.view(B, 1, S, 1).float()
+        j = torch.arange(L, device=q.device).view(1, 1, 1, L).float()
+        dist = (i - j).clamp(min=0)
+        s = s - r1.float().view(1, H, 1, 1) * torch.log1p(
+            r2.float().view(1, H, 1, 1) * dist)
+        vis = (j <= i) & ((i - j < window) | (j < keep_first))
+        s = s.masked_fill(~vis, float("-inf"))
+        p = torch.nan_to_num(torch.softmax(s, dim=-1))
+        out = torch.einsum("bhsl,blhd->bshd", p, v)
+    out = out.reshape(B, S, H * Dv)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())
+    return out.to(out_dtype)
+
+
+def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps, state,
+                     positions, seq_ids, kv_heads, dim, vdim,
+                     out_dtype=torch.float32):
+    """Delta-rule recurrence with a per-key-channel decay, carried state
+    (slots, H, dim, vdim) fp32. qkv (B,S,2*G*dim + H*vdim) holds the
+    convolved+activated q|k|v; beta (B,S,H) and a (B,S,H*dim), gate
+    (B,S,H*vdim) are pre-activation projections. Per token and head:
+      S <- diag(decay) S ; u = beta (v - S^T k) ; S <- S + k u^T ; o = S^T q
+    followed by o / rms(o) * norm_w * sigmoid(gate)."""
+    B, S, _ = qkv.shape
+    G, D, Dv = kv_heads, dim, vdim
+    H = beta.shape[-1]
+    rep = H // G
+    f = qkv.float()
+    q = f[..., :G * D].view(B, S, G, D)
+    k = f[..., G * D:2 * G * D].view(B, S, G, D)
+    v = f[..., 2 * G * D:].view(B, S, H, Dv)
+    q = q * torch.rsqrt((q * q).sum(-1, keepdim=True) + 1e-6) * (D ** -0.5)
+    k = k * torch.rsqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+    q = q.repeat_interleave(rep, dim=2)
+    k = k.repeat_interleave(rep, dim=2)
+    bt = torch.sigmoid(beta.float())
+    dt = torch.nn.functional.softplus(a.float() + dt_bias.float()).view(B, S, H, D)
+    decay = torch.exp(-torch.exp(a_log.float()).view(1, 1, H, 1) * dt)
+    out = torch.zeros(B, S, H, Dv, dtype=torch.float32, device=qkv.device)
+    n_valid, p0s = _row_extent(positions)
+    for b in range(B):
+        slot = int(seq_ids[b])
+        n = int(n_valid[b])
+        if slot < 0 or n == 0:
+            continue
+        St = state[slot].float() if int(p0s[b]) > 0 else torch.zeros_like(state[slot], dtype=torch.float32)
+        for t in range(n):
+            St = decay[b, t].unsqueeze(-1) * St
+            u = bt[b, t].unsqueeze(-1) * (v[b, t] - torch.einsum("hdv,hd->hv", St, k[b, t]))
+            St = St + k[b, t].unsqueeze(-1) * u.unsqueeze(1)
+            out[b, t] = torch.einsum("hdv,hd->hv", St, q[b, t])
+        state[slot] = St.to(state.dtype)
+    out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps) * norm_w.float()
+    out = out.reshape(B, S, H * Dv) * torch.sigmoid(gate.float())
+    return out.to(out_dtype)
+
+
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    return cap * torch.tanh(logits.float() / cap)

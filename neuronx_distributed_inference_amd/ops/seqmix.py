@@ -1,0 +1,292 @@
+"""Sequence-mixing ops of hybrid (windowed attention + linear recurrence)
+models: dispatch between the gfx950 kernels of ``csrc/seqmix.hip`` and the
+torch references in ``ops.ref`` (CPU execution and numerics oracle).
+
+The kernels live in their own small shared library ``_nxdi_seqmix.so`` with
+a C ABI, loaded through ctypes: it has no torch headers, so a fresh checkout
+compiles it with one ``hipcc`` call in seconds and a model that needs only
+these ops never waits for the large extension. Launches go to torch's
+current HIP stream. On a GPU tensor the library is required — there is no
+silent fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+import threading
+from typing import Optional
+
+import torch
+
+from neuronx_distributed_inference_amd.ops import ref
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "_nxdi_seqmix.so")
+SRC_PATH = os.path.join(_HERE, "csrc", "seqmix.hip")
+HIPCC_FLAGS = [
+    "-O3", "-std=c++17", "--offload-arch=gfx950", "-shared", "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+_lib = None
+_lib_error: Optional[BaseException] = None
+_lock = threading.Lock()
+
+
+def build(force: bool = False) -> str:
+    """Compile the library in-tree (cross-compiles without a GPU)."""
+    if not force and os.path.exists(LIB_PATH) and \
+            os.path.getmtime(LIB_PATH) >= os.path.getmtime(SRC_PATH):
+        return LIB_PATH
+    hipcc = os.environ.get("HIPCC") or (
+        "/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else "hipcc")
+    tmp = LIB_PATH + ".%d.tmp" % os.getpid()
+    subprocess.run([hipcc] + HIPCC_FLAGS + ["-o", tmp, SRC_PATH], check=True,
+                   stdout=subprocess.DEVNULL, stderr=subprocess.PIPE)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+def _load():
+    global _lib, _lib_error
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        try:
+            build()
+            _lib = ctypes.CDLL(LIB_PATH)
+        except BaseException as e:  # noqa: BLE001
+            _lib_error = e
+            raise RuntimeError(
+                "sequence-mixing op called on a GPU tensor but _nxdi_seqmix.so "
+                f"could not be built/loaded: {e!r}") from e
+    return _lib
+
+
+def library_available() -> bool:
+    try:
+        _load()
+        return True
+    except RuntimeError:
+        return False
+
+
+def _p(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _is_bf16(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return 1
+    if t.dtype == torch.float32:
+        return 0
+    raise TypeError(f"seqmix ops take float32 or bfloat16, got {t.dtype}")
+
+
+def _check(rc: int, name: str):
+    if rc != 0:
+        raise RuntimeError(f"{name}: launch failed / unsupported shape (code {rc})")
+
+
+def _i32(t: torch.Tensor) -> torch.Tensor:
+    return t if t.dtype == torch.int32 and t.is_contiguous() else t.to(torch.int32).contiguous()
+
+
+def _f32(t: torch.Tensor) -> torch.Tensor:
+    return t if t.dtype == torch.float32 and t.is_contiguous() else t.float().contiguous()
+
+
+def _rows_view(t: torch.Tensor):
+    """(..., C) tensor whose leading dims collapse to rows with one stride
+    (a column slice of a fused GEMM output qualifies): returns row stride."""
+    assert t.stride(-1) == 1, "innermost dim must be contiguous"
+    if t.dim() == 3:
+        assert t.stride(0) == t.stride(1) * t.shape[1], "rows must be uniformly strided"
+        return t.stride(1)
+    return t.stride(0)
+
+
+class StepLayout:
+    """Per-step ragged-batch descriptors shared by every layer's kernels:
+    int32 positions (B,S), state slots (B,), valid-token counts (B,)."""
+
+    def __init__(self, positions: torch.Tensor, seq_ids: torch.Tensor):
+        self.positions = _i32(positions)
+        self.seq_ids = _i32(seq_ids)
+        self.nvalid = (self.positions >= 0).sum(-1).to(torch.int32)
+
+
+# ----------------------------------------------------------------------
+def layer_norm(x, weight, eps: float, out_dtype: torch.dtype):
+    """Bias-free LayerNorm of an fp32 stream, fp32 statistics."""
+    if x.is_cuda:
+        lib = _load()
+        x = _f32(x)
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        C = x.shape[-1]
+        _check(lib.nx_layer_norm(_p(x), _p(_f32(weight)), _p(out), _is_bf16(out),
+                                 ctypes.c_long(x.numel() // C), C,
+                                 ctypes.c_float(eps), _stream()), "layer_norm")
+        return out
+    return ref.layer_norm(x, weight, eps, out_dtype)
+
+
+def short_conv(x, w, tail, step: StepLayout, activation: str = "none",
+               residual: bool = False, out_dtype=torch.float32):
+    """Depthwise causal conv over time with a carried tail (see
+    ref.short_conv). Does not advance the tail: call short_conv_commit."""
+    if x.is_cuda:
+        lib = _load()
+        x = x.contiguous()
+        B, S, C = x.shape
+        y = torch.empty(B, S, C, dtype=out_dtype, device=x.device)
+        _check(lib.nx_short_conv(
+            _p(x), _is_bf16(x), _p(_f32(w)), _p(tail), _p(step.positions),
+            _p(step.seq_ids), _p(y), _is_bf16(y), B, S, C, w.shape[1],
+            int(activation == "silu"), int(residual), _stream()), "short_conv")
+        return y
+    return ref.short_conv(x, w, tail, step.positions, step.seq_ids,
+                          activation, residual, out_dtype)
+
+
+def short_conv_commit(x, tail, step: StepLayout):
+    if x.is_cuda:
+        lib = _load()
+        x = x.contiguous()
+        B, S, C = x.shape
+        assert tail.dtype == torch.float32 and tail.is_contiguous()
+        _check(lib.nx_short_conv_commit(
+            _p(x), _is_bf16(x), _p(tail), _p(step.positions), _p(step.seq_ids),
+            _p(step.nvalid), B, S, C, tail.shape[1], _stream()), "short_conv_commit")
+        return
+    ref.short_conv_commit(x, tail, step.positions, step.seq_ids)
+
+
+def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping):
+    """Scatter k_new (N, G*Dk) / v_new (N, G*Dv) rows (row-strided views
+    allowed) into paged caches (blocks, block, G, D*)."""
+    if k_cache.is_cuda:
+        lib = _load()
+        N = k_new.shape[0]
+        GDk = k_cache.shape[2] * k_cache.shape[3]
+        GDv = v_cache.shape[2] * v_cache.shape[3]
+        assert k_new.shape[1] == GDk and v_new.shape[1] == GDv
+        assert k_new.dtype == k_cache.dtype == v_new.dtype == v_cache.dtype
+        assert k_new.stride(1) == 1 and v_new.stride(1) == 1
+        _check(lib.nx_paged_kv_write(
+            _p(k_cache), _p(v_cache), _p(k_new), ctypes.c_long(k_new.stride(0)),
+            _p(v_new), ctypes.c_long(v_new.stride(0)), _is_bf16(k_cache),
+            _p(_i32(slot_mapping)), ctypes.c_long(N), GDk, GDv,
+            ctypes.c_long(k_cache.shape[0] * k_cache.shape[1]), _stream()),
+            "paged_kv_write")
+        return
+    G = k_cache.shape[2]
+    ref.paged_kv_write(k_cache, v_cache, k_new.reshape(k_new.shape[0], G, -1),
+                       v_new.reshape(v_new.shape[0], G, -1), slot_mapping)
+
+
+def window_bias_attention(q, k_cache, v_cache, step: StepLayout, block_table,
+                          r1, r2, scale: float, window: int, keep_first: int,
+                          num_heads: int, gate=None, out_dtype=None):
+    """q (B,S,H*Dk) (row-strided view allowed) against the paged cache ->
+    (B,S,H*Dv); see ref.window_bias_attention for the masking and bias."""
+    B, S = q.shape[0], q.shape[1]
+    H = num_heads
+    G, Dk = k_cache.shape[2], k_cache.shape[3]
+    Dv = v_cache.shape[3]
+    out_dtype = out_dtype or q.dtype
+    if q.is_cuda:
+        lib = _load()
+        out = torch.empty(B, S, H * Dv, dtype=out_dtype, device=q.device)
+        bt = _i32(block_table)
+        _check(lib.nx_window_attn(
+            _p(q), ctypes.c_long(_rows_view(q)), _p(k_cache), _p(v_cache),
+            _p(step.positions), _p(bt), bt.shape[1], _p(_f32(r1)), _p(_f32(r2)),
+            _p(gate), ctypes.c_long(0 if gate is None else _rows_view(gate)),
+            _p(out), _is_bf16(q), _is_bf16(out), B, S, H, G, Dk, Dv,
+            k_cache.shape[1], ctypes.c_float(scale), int(window), int(keep_first),
+            _stream()), "window_bias_attention")
+        return out
+    return ref.window_bias_attention(
+        q.reshape(B, S, H, Dk), k_cache, v_cache, step.positions, block_table,
+        r1, r2, scale, window, keep_first, gate=gate, out_dtype=out_dtype)
+
+
+def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps: float,
+                     state, step: StepLayout, kv_heads: int, dim: int, vdim: int,
+                     out_dtype=torch.float32):
+    """Gated delta-rule recurrence over the step's tokens, state carried in
+    `state` (slots, H, dim, vdim) fp32; see ref.gated_delta_rule."""
+    if qkv.is_cuda:
+        lib = _load()
+        B, S = qkv.shape[0], qkv.shape[1]
+        H = beta.shape[-1]
+        assert qkv.dtype == torch.float32 and state.dtype == torch.float32
+        assert beta.dtype == a.dtype == gate.dtype == out_dtype
+        out = torch.empty(B, S, H * vdim, dtype=out_dtype, device=qkv.device)
+        _check(lib.nx_gated_delta(
+            _p(qkv), ctypes.c_long(_rows_view(qkv)), _p(beta),
+            ctypes.c_long(_rows_view(beta)), _p(a), ctypes.c_long(_rows_view(a)),
+            _p(gate), ctypes.c_long(_rows_view(gate)), _p(_f32(dt_bias)),
+            _p(_f32(a_log)), _p(_f32(norm_w)), ctypes.c_float(eps), _p(state),
+            _p(step.positions), _p(step.seq_ids), _p(step.nvalid), _p(out),
+            _is_bf16(beta), B, S, H, kv_heads, dim, vdim, _stream()),
+            "gated_delta_rule")
+        return out
+    return ref.gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps,
+                                state, step.positions, step.seq_ids, kv_heads,
+                                dim, vdim, out_dtype)
+
+
+def softcap(logits, cap: float):
+    """cap * tanh(logits / cap) in fp32."""
+    if logits.is_cuda:
+        lib = _load()
+        x = logits.contiguous()
+        out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        _check(lib.nx_softcap(_p(x), _is_bf16(x), _p(out), ctypes.c_long(x.numel()),
+                              ctypes.c_float(cap), _stream()), "softcap")
+        return out
+    return ref.softcap(logits, cap)
+
+
+def residual_add(x, a, sa: float = 1.0, b=None, sb: float = 1.0):
+    """In place on the fp32 stream: x += sa*a (+ sb*b)."""
+    if x.is_cuda:
+        lib = _load()
+        assert x.dtype == torch.float32 and x.is_contiguous()
+        a = a.contiguous()
+        if b is not None:
+            b = b.contiguous()
+            assert b.dtype == a.dtype
+        _check(lib.nx_residual_add(_p(x), _p(a), ctypes.c_float(sa), _p(b),
+                                   ctypes.c_float(sb), _is_bf16(a),
+                                   ctypes.c_long(x.numel()), _stream()), "residual_add")
+        return x
+    x.add_(a.float(), alpha=sa)
+    if b is not None:
+        x.add_(b.float(), alpha=sb)
+    return x
+
+
+def gelu_tanh_mul_fused(gate_up):
+    """(rows, 2I) [gate | up] -> gelu_tanh(gate) * up."""
+    I = gate_up.shape[-1] // 2
+    if gate_up.is_cuda:
+        lib = _load()
+        gu = gate_up.contiguous()
+        out = torch.empty(gu.shape[:-1] + (I,), dtype=gu.dtype, device=gu.device)
+        _check(lib.nx_gelu_mul(_p(gu), _p(out), _is_bf16(gu),
+                               ctypes.c_long(gu.numel() // (2 * I)), I, _stream()),
+               "gelu_tanh_mul_fused")
+        return out
+    g, u = gate_up.float().chunk(2, dim=-1)
+    return ref.gelu_tanh_mul(g, u).to(gate_up.dtype)

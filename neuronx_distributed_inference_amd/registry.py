@@ -66,6 +66,11 @@ _REGISTRY: Dict[str, Tuple[str, str, str]] = {
         "Qwen3MoeInferenceConfig",
         "Qwen3MoeForCausalLM",
     ),
+    "nabelix": (
+        "neuronx_distributed_inference_amd.models.nabelix.modeling_nabelix",
+        "NabelixInferenceConfig",
+        "NabelixForCausalLM",
+    ),
     # conditional-generation families (multimodal / speech): resolved for
     # programmatic use; the CLI's causal-lm run path does not drive these
     "whisper": (
@@ -122,3 +127,25 @@ def get_model_classes(model_type: str) -> Tuple[Type, Type]:
     mod_name, cfg_name, mdl_name = _REGISTRY[model_type]
     mod = importlib.import_module(mod_name)
     return getattr(mod, cfg_name), getattr(mod, mdl_name)
+
+
+def model_type_from_config(model_path: str) -> str:
+    """Resolve the registry key from a checkpoint's ``config.json``:
+    ``model_type`` (HF convention) or ``architecture`` / ``architectures``
+    (matched case-insensitively, with a trailing ForCausalLM dropped)."""
+    import json
+    import os
+
+    with open(os.path.join(model_path, "config.json")) as f:
+        cfg = json.load(f)
+    cands = [cfg.get("model_type"), cfg.get("architecture")]
+    cands += list(cfg.get("architectures") or [])
+    for c in cands:
+        if not c:
+            continue
+        key = str(c).lower()
+        for k in (key, key.replace("forcausallm", "")):
+            if k in _REGISTRY:
+                return k
+    raise KeyError(f"no registered model for config {cands}; "
+                   f"available: {available_model_types()}")

@@ -78,6 +78,10 @@ class ServingEngine:
             self.allocator = BlockAllocator(self.kv_mgr.num_blocks)
             self.prefix_cache = PrefixCache(self.allocator, self.block_size)
             self.max_blocks = (ec.max_length + self.block_size - 1) // self.block_size
+        # content-addressed KV pages can stand in for a prompt prefix only if
+        # KV is the whole context; recurrent state is not page-addressable
+        self.prefix_caching = self.paged and not getattr(
+            self.kv_mgr, "has_recurrent_state", False)
         self.free_slots = list(range(self.max_slots))[::-1]
         self.active: Dict[int, Request] = {}    # slot -> request
         self.queue: Deque[Request] = collections.deque()
@@ -196,7 +200,7 @@ class ServingEngine:
 
     def _prefill_chunk(self, req: Request):
         S = req.prompt.shape[0]
-        if self.paged and req.prefill_done == 0 and not req.blocks:
+        if self.prefix_caching and req.prefill_done == 0 and not req.blocks:
             # prefix-cache hit: shared FULL blocks skip their prefill
             req.blocks = self.prefix_cache.match(req.prompt.tolist())
             req.n_cached = len(req.blocks) * self.block_size
@@ -367,19 +371,25 @@ class ServingEngine:
         if len(req.output) >= req.max_new_tokens or (
             self.eos is not None and tok == self.eos
         ):
-            req.done = True
-            req.t_finish = time.monotonic()
-            self.active.pop(req.slot)
-            self.free_slots.append(req.slot)
-            self.finished[req.req_id] = req
-            if self.paged and req.blocks:
+            self._release(req)
+
+    def _release(self, req: Request):
+        """Retire a request: its state slot and KV pages go back to the
+        pools (a later request reuses them)."""
+        req.done = True
+        req.t_finish = time.monotonic()
+        self.active.pop(req.slot)
+        self.free_slots.append(req.slot)
+        self.finished[req.req_id] = req
+        if self.paged and req.blocks:
+            if self.prefix_caching:
                 # register the prompt's FULL blocks for future prefix hits,
                 # then drop this request's references
                 n_prompt_blocks = req.prompt.shape[0] // self.block_size
                 self.prefix_cache.insert(req.prompt.tolist(),
                                          req.blocks[:n_prompt_blocks])
-                self.allocator.deref(req.blocks)
-                req.blocks = []
+            self.allocator.deref(req.blocks)
+            req.blocks = []
 
     # ------------------------------------------------------------------
     def step(self):
@@ -404,7 +414,9 @@ class ServingEngine:
                             if self.active[s] is not r
                             and self.active[s].prefill_done
                             >= self.active[s].prompt.shape[0]]
-                if self.mixed_chunking and decoding and not self.paged:
+                if self.mixed_chunking and decoding and (
+                        not self.paged or r.prefill_done > 0
+                        or not self.prefix_caching):
                     self._mixed_step(r, decoding)
                 else:
                     self._prefill_chunk(r)
@@ -423,29 +435,15 @@ class ServingEngine:
         hi = S if self.chunk_size is None else min(S, lo + self.chunk_size)
         L = hi - lo
         B = self.batch
-        ids = torch.zeros(B, L, dtype=torch.long, device=self.device)
-        pos = torch.full((B, L), -1, dtype=torch.long, device=self.device)
-        seq_ids = torch.full((B,), -1, dtype=torch.long, device=self.device)
-        ids[0, :L] = pre.prompt[lo:hi].to(self.device)
-        pos[0, :L] = torch.arange(lo, hi, device=self.device)
-        seq_ids[0] = pre.slot
-        reqs = [pre] + [self.active[s] for s in decode_slots]
-        for i, slot in enumerate(decode_slots, start=1):
-            if i >= B:
-                decode_slots = decode_slots[: i - 1]
-                reqs = reqs[: i]
-                break
+        decode_slots = decode_slots[: B - 1]
+        rows = [(pre, pre.prompt[lo:hi], lo)]
+        for slot in decode_slots:
             r = self.active[slot]
-            ids[i, 0] = r.last_token
-            pos[i, 0] = r.pos
-            seq_ids[i] = slot
-        self._set_adapters(reqs)
-        out = self.model(ids, None, pos, seq_ids, None,
-                         phase="token_generation")
-        toks = out.logits if out.logits is not None else out.tokens
+            rows.append((r, torch.tensor([r.last_token]), r.pos))
+        toks = self._run_rows(rows)
         if toks.dim() > 2:
             toks = toks.argmax(-1)
-        toks = toks.view(B, -1)
+        toks = toks.view(len(rows), -1)
         pre.prefill_done = hi
         host = toks.cpu()
         if hi == S:  # chunk completes the prompt: emit its first token
@@ -470,6 +468,71 @@ class ServingEngine:
             if self.on_token is not None:
                 self.on_token(r.req_id, tok)
             self._maybe_finish(r, tok)
+
+    # ------------------------------------------------------------------
+    def _run_rows(self, rows):
+        """One model step over ragged rows [(request, tokens (n,), first
+        position)]: the batch is right-padded with position -1 / seq_id -1
+        (the pad-skip invariant keeps pads out of cache, state and
+        attention); paged engines grow each row's block chain first.
+        Returns the model output over the padded (B, L) batch — per-position
+        logits, or greedy tokens when the sampler runs on device."""
+        B = len(rows)
+        L = max(int(t.shape[0]) for _, t, _ in rows)
+        ids = torch.zeros(B, L, dtype=torch.long)
+        pos = torch.full((B, L), -1, dtype=torch.long)
+        seq = torch.full((B,), -1, dtype=torch.long)
+        for i, (r, toks, lo) in enumerate(rows):
+            n = int(toks.shape[0])
+            ids[i, :n] = toks
+            pos[i, :n] = torch.arange(lo, lo + n)
+            seq[i] = r.slot
+        reqs = [r for r, _, _ in rows]
+        self._set_adapters(reqs)
+        kw = {}
+        if self.paged:
+            for r, toks, lo in rows:
+                self._ensure_blocks(r, lo + int(toks.shape[0]) - 1)
+            kw["block_table"] = self._block_table(reqs)
+        out = self.model(ids.to(self.device), None, pos.to(self.device),
+                         seq.to(self.device), None, phase="token_generation", **kw)
+        return out.logits if out.logits is not None else out.tokens
+
+    def admit(self, prompt_ids: Optional[torch.Tensor] = None) -> Request:
+        """Take a state slot for a request outside the queue (externally
+        driven steps). Raises when every slot is live."""
+        if not self.free_slots:
+            raise RuntimeError("no free sequence slot")
+        rid = self._next_id
+        self._next_id += 1
+        prompt = torch.zeros(0, dtype=torch.long) if prompt_ids is None \
+            else prompt_ids.view(-1).cpu()
+        req = Request(rid, prompt)
+        req.t_submit = time.monotonic()
+        req.slot = self.free_slots.pop()
+        self.active[req.slot] = req
+        return req
+
+    def forced_step(self, parts):
+        """Run one engine step on GIVEN tokens instead of sampled ones:
+        `parts` is [(request, tokens (n,))], each request's next tokens —
+        prompt portions and single tokens side by side in one batch. Cache,
+        state and positions advance exactly as in generation. Returns the
+        per-position logits (B, L, vocab) of the padded batch."""
+        self._drain_inflight(0)
+        rows = [(r, t.view(-1).cpu().long(), r.pos) for r, t in parts]
+        logits = self._run_rows(rows)
+        if logits.dim() != 3:
+            raise RuntimeError("forced_step needs host-visible logits "
+                               "(no on-device sampler, or output_logits=True)")
+        for r, t, _ in rows:
+            r.pos += int(t.shape[0])
+            r.prefill_done = r.pos
+        return logits
+
+    def release(self, req: Request):
+        self._drain_inflight(0)
+        self._release(req)
 
     def run(self, max_steps: int = 100000) -> Dict[int, List[int]]:
         steps = 0
