@@ -68,7 +68,146 @@ def parse_args():
     p.add_argument("--spec", action="store_true",
                    help="fused speculative decoding: --model target + 1b draft, spec-len 5")
     p.add_argument("--spec-len", type=int, default=5)
+    p.add_argument("--hybrid", action="store_true",
+                   help="Nabelix (windowed attention + gated delta rule) prefill/decode "
+                        "throughput beside Llama at equal width/depth/ff/vocab")
+    p.add_argument("--hybrid-sizes", default="2048,4096",
+                   help="comma-separated layer widths for --hybrid")
+    p.add_argument("--hybrid-layers", type=int, default=4)
+    p.add_argument("--hybrid-prompt", type=int, default=4096)
     return p.parse_args()
+
+
+HYBRID_SIZES = {
+    256: (2, 1, 512),
+    # width: heads, kv_heads, ff  (head size 128 everywhere)
+    1024: (8, 2, 4096),
+    2048: (16, 4, 8192),
+    4096: (32, 8, 14336),
+}
+
+
+def run_hybrid_bench(args):
+    """Prefill tokens/s (one prompt of --hybrid-prompt tokens) and decode
+    tokens/s (--batch-per-gpu sequences at --ctx, hipGraph-captured step) of
+    Nabelix and of Llama with the same width, depth, feed-forward size,
+    head geometry and vocabulary; random weights, synthetic tokens. Prints
+    one JSON line per (model, width)."""
+    on_gpu = torch.cuda.is_available()
+    device = torch.device("cuda:0" if on_gpu else "cpu")
+    from neuronx_distributed_inference_amd.config import (
+        EngineConfig, OnDeviceSamplingConfig,
+    )
+    from neuronx_distributed_inference_amd.models.llama.modeling_llama import (
+        LlamaForCausalLM, LlamaInferenceConfig,
+    )
+    from neuronx_distributed_inference_amd.models.nabelix.modeling_nabelix import (
+        NabelixForCausalLM, NabelixInferenceConfig,
+    )
+
+    dtype = "bfloat16" if on_gpu else "float32"
+    B, ctx, steps, warmup = args.batch_per_gpu, args.ctx, args.steps, args.warmup
+    P = args.hybrid_prompt
+    L, V = args.hybrid_layers, 32000
+    max_len = max(P, ctx + steps + warmup + 8)
+
+    def sync():
+        if on_gpu:
+            torch.cuda.synchronize()
+
+    def build(kind, width, batch):
+        H, G, ff = HYBRID_SIZES[width]
+        ec = EngineConfig(
+            batch_size=batch, max_batch_size=batch, seq_len=max_len, max_length=max_len,
+            max_context_length=P, torch_dtype=dtype, tp_degree=1,
+            on_device_sampling_config=OnDeviceSamplingConfig(top_k=1),
+            enable_hip_graphs=not args.no_graphs, fused_qkv=True, fused_gate_up=True,
+            enable_batch_bucketing=False, pa_block_size=64,
+        )
+        if kind == "llama":
+            cfg = LlamaInferenceConfig(
+                neuron_config=ec, hidden_size=width, intermediate_size=ff,
+                num_hidden_layers=L, num_attention_heads=H, num_key_value_heads=G,
+                head_dim=128, vocab_size=V, max_position_embeddings=max_len * 2,
+                rms_norm_eps=1e-5, rope_theta=500000.0, hidden_act="silu",
+                tie_word_embeddings=False)
+            cls = LlamaForCausalLM
+        else:
+            layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff}, "mixer": {
+                "left": {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128,
+                         "scale": 128 ** -0.5, "mask": {"size": 1024, "keep_first": 4}},
+                "right": {"heads": H, "kv_heads": H, "dim": 128, "vdim": 128, "conv": 4,
+                          "decay_rank": 64, "gate_rank": 64},
+                "left_scale": 1.0, "right_scale": 1.0}}
+            cfg = NabelixInferenceConfig(
+                neuron_config=ec, architecture="Nabelix", width=width, vocab=V,
+                layers=[layer] * L, canon={"taps": 4}, norm={"eps": 1e-5},
+                loop={"start": 0, "stop": 0, "times": 1}, logit_softcap=30.0)
+            cls = NabelixForCausalLM
+        torch.manual_seed(1234)
+        if on_gpu:
+            with torch.device(device):
+                m = cls(cfg).eval()
+        else:
+            m = cls(cfg).eval()
+        with torch.no_grad():
+            for p in m.parameters():
+                if p.dim() >= 2 and p.requires_grad:   # caches/state do not
+                    p.normal_(0, 0.02)
+        m.reset()
+        m.enable_submodels()
+        return m
+
+    for width in [int(x) for x in args.hybrid_sizes.split(",")]:
+        for kind in ("llama", "nabelix"):
+            with torch.inference_mode():
+                # ---- prefill: one prompt, three timed repetitions
+                m = build(kind, width, 1)
+                ids = torch.randint(0, V, (1, P), device=device)
+                pos = torch.arange(P, device=device).view(1, P)
+                sid = torch.zeros(1, dtype=torch.long, device=device)
+                for _ in range(2):
+                    m.reset()
+                    m(input_ids=ids, position_ids=pos, seq_ids=sid)
+                sync()
+                t0 = time.perf_counter()
+                for _ in range(3):
+                    m.kv_cache_populated = False
+                    m(input_ids=ids, position_ids=pos, seq_ids=sid)
+                sync()
+                prefill_s = (time.perf_counter() - t0) / 3
+                del m
+                # ---- decode: B sequences at ctx
+                m = build(kind, width, B)
+                if on_gpu and not args.no_graphs:
+                    m.warmup()
+                ids = torch.randint(0, V, (B, ctx), device=device)
+                pos = torch.arange(ctx, device=device).view(1, ctx).expand(B, ctx).contiguous()
+                sid = torch.arange(B, device=device)
+                tok = m(input_ids=ids, position_ids=pos, seq_ids=sid).tokens.view(-1, 1)
+                pos_t = torch.full((B, 1), ctx, device=device, dtype=torch.long)
+                for _ in range(warmup):
+                    tok = m(input_ids=tok, position_ids=pos_t, seq_ids=sid).tokens.view(-1, 1)
+                    pos_t.add_(1)
+                sync()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    tok = m(input_ids=tok, position_ids=pos_t, seq_ids=sid).tokens.view(-1, 1)
+                    pos_t.add_(1)
+                sync()
+                decode_s = (time.perf_counter() - t0) / steps
+                del m
+                if on_gpu:
+                    torch.cuda.empty_cache()
+            print(json.dumps({
+                "bench": "hybrid", "model": kind, "width": width, "layers": L,
+                "dtype": dtype, "data": "synthetic, random-init",
+                "prefill_tokens": P, "prefill_ms": round(prefill_s * 1e3, 3),
+                "prefill_tok_s": round(P / prefill_s, 1),
+                "decode_batch": B, "decode_ctx": ctx,
+                "decode_ms_per_step": round(decode_s * 1e3, 3),
+                "decode_tok_s": round(B / decode_s, 1),
+            }), flush=True)
 
 
 def run_spec_bench(args):
@@ -181,6 +320,8 @@ def main():
     args = parse_args()
     if args.spec:
         return run_spec_bench(args)
+    if args.hybrid:
+        return run_hybrid_bench(args)
     world = int(os.environ.get("WORLD_SIZE", 1))
     rank = int(os.environ.get("RANK", 0))
     local_rank = int(os.environ.get("LOCAL_RANK", 0))

@@ -260,8 +260,11 @@ class NabelixModel(DecoderModel):
             if self.kv_mgr.num_blocks < self.kv_mgr.state.num_slots * M:
                 raise RuntimeError(
                     "the page pool is smaller than slots x max_length: pass a block_table")
-            block_table = seq_ids.long().clamp(min=0).view(B, 1) * M + torch.arange(
-                M, device=position_ids.device).view(1, M)
+            sid = seq_ids.long().view(B, 1)
+            block_table = torch.where(
+                sid >= 0,
+                sid * M + torch.arange(M, device=position_ids.device).view(1, M),
+                torch.full_like(sid, -1))     # pad rows own no pages
         return block_table
 
     def prepare_hidden(self, h):

@@ -157,6 +157,7 @@ template <typename T, typename TOut>
 __global__ void __launch_bounds__(ATT_WAVES * WAVE)
 window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ kc,
                    const T* __restrict__ vc, const int* __restrict__ pos,
+                   const int* __restrict__ seq,
                    const int* __restrict__ btab, int max_blocks, const float* __restrict__ r1,
                    const float* __restrict__ r2, const T* __restrict__ gate, long gstride,
                    TOut* __restrict__ out, long ntok, int H, int G, int Dk, int Dv,
@@ -168,7 +169,7 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
     const bool live = wid < ntok * H;
     const long tok = live ? wid / H : 0;
     const int h = live ? (int)(wid % H) : 0;
-    const int i = live ? pos[tok] : -1;
+    const int i = (live && seq[tok / S] >= 0) ? pos[tok] : -1;
     float* myq = qs + wv * Dk;
     if (i >= 0) {
         const T* qp = q + tok * qstride + (long)h * Dk;
@@ -195,7 +196,8 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
         long slot = 0;
         if (m < n) {
             const int j = m < nfirst ? m : lo + (m - nfirst);
-            slot = (long)bt[j / bsz] * bsz + (j % bsz);
+            const int blk = bt[j / bsz];
+            slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);   // unmapped page: row 0, never hit by a live row
             const T* kp = kc + slot * krow + (long)g * Dk;
             float dot = 0.f;
             if constexpr (sizeof(T) == 2) {
@@ -487,7 +489,7 @@ int nx_paged_kv_write(void* kc, void* vc, const void* k, long kstride, const voi
 }
 
 int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, const int* pos,
-                   const int* btab, int max_blocks, const float* r1, const float* r2,
+                   const int* seq, const int* btab, int max_blocks, const float* r1, const float* r2,
                    const void* gate, long gstride, void* out, int io_bf16, int out_bf16,
                    int B, int S, int H, int G, int Dk, int Dv, int bsz, float scale, int window,
                    int keep, hipStream_t st) {
@@ -498,7 +500,7 @@ int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, 
     dim3 grid((unsigned)((waves + ATT_WAVES - 1) / ATT_WAVES)), block(ATT_WAVES * WAVE);
     const size_t sh = (size_t)ATT_WAVES * Dk * sizeof(float);
 #define WA(T, TO) window_attn_kernel<T, TO><<<grid, block, sh, st>>>( \
-        (const T*)q, qstride, (const T*)kc, (const T*)vc, pos, btab, max_blocks, r1, r2, \
+        (const T*)q, qstride, (const T*)kc, (const T*)vc, pos, seq, btab, max_blocks, r1, r2, \
         (const T*)gate, gstride, (TO*)out, ntok, H, G, Dk, Dv, bsz, S, scale, window, keep)
     if (io_bf16 && out_bf16) WA(bf16, bf16);
     else if (io_bf16) WA(bf16, float);

@@ -209,7 +209,8 @@ def window_bias_attention(q, k_cache, v_cache, step: StepLayout, block_table,
         bt = _i32(block_table)
         _check(lib.nx_window_attn(
             _p(q), ctypes.c_long(_rows_view(q)), _p(k_cache), _p(v_cache),
-            _p(step.positions), _p(bt), bt.shape[1], _p(_f32(r1)), _p(_f32(r2)),
+            _p(step.positions), _p(step.seq_ids), _p(bt), bt.shape[1],
+            _p(_f32(r1)), _p(_f32(r2)),
             _p(gate), ctypes.c_long(0 if gate is None else _rows_view(gate)),
             _p(out), _is_bf16(q), _is_bf16(out), B, S, H, G, Dk, Dv,
             k_cache.shape[1], ctypes.c_float(scale), int(window), int(keep_first),
