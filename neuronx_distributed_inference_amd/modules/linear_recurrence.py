@@ -53,7 +53,7 @@ class GatedDeltaRule(nn.Module):
 
     def state_shapes(self):
         return {"conv": self.conv.state_shape(),
-                "mem": (self.num_heads, self.dim, self.vdim)}
+                "mem": (self.num_heads, self.vdim, self.dim)}   # stored transposed
 
     def forward(self, qkv: torch.Tensor, beta: torch.Tensor, a_low: torch.Tensor,
                 g_low: torch.Tensor, states, key: str,

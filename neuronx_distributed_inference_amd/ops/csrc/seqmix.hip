@@ -45,22 +45,38 @@ DEV float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
 DEV float softplusf_(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
 // ---------------------------------------------------------------- LayerNorm
-// one wave per row; mean, then variance of the deviations (both fp32)
+// one 256-thread workgroup per row; mean, then variance of the deviations
+// (both fp32); the row is re-read from cache, not kept in registers, so any
+// width works
+#define LN_THREADS 256
+
+DEV float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & (WAVE - 1), wv = threadIdx.x / WAVE;
+    __syncthreads();                       // red may still be read by the previous call
+    if (lane == 0) red[wv] = v;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < LN_THREADS / WAVE; ++i) t += red[i];
+    return t;
+}
+
 template <typename TOut>
-__global__ void layer_norm_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                  TOut* __restrict__ out, long rows, int C, float eps) {
-    const int lane = threadIdx.x & (WAVE - 1);
-    const long row = (long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-    if (row >= rows) return;
+__global__ void __launch_bounds__(LN_THREADS)
+layer_norm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                  TOut* __restrict__ out, long rows, int C, float eps) {
+    __shared__ float red[LN_THREADS / WAVE];
+    const long row = blockIdx.x;
     const float* xr = x + row * C;
     float s = 0.f;
-    for (int c = lane; c < C; c += WAVE) s += xr[c];
-    const float mean = wave_sum(s) / C;
+    for (int c = threadIdx.x; c < C; c += LN_THREADS) s += xr[c];
+    const float mean = block_sum(s, red) / C;
     float v = 0.f;
-    for (int c = lane; c < C; c += WAVE) { float d = xr[c] - mean; v += d * d; }
-    const float inv = 1.f / sqrtf(wave_sum(v) / C + eps);
+    for (int c = threadIdx.x; c < C; c += LN_THREADS) { float d = xr[c] - mean; v += d * d; }
+    const float inv = 1.f / sqrtf(block_sum(v, red) / C + eps);
     TOut* o = out + row * C;
-    for (int c = lane; c < C; c += WAVE) stf<TOut>(o + c, (xr[c] - mean) * inv * w[c]);
+    for (int c = threadIdx.x; c < C; c += LN_THREADS) stf<TOut>(o + c, (xr[c] - mean) * inv * w[c]);
 }
 
 // ------------------------------------------------------------- short conv
@@ -261,57 +277,65 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
 }
 
 // ------------------------------------------------------- gated delta rule
-// One workgroup per (row, head); thread j owns column j of the (D x Dv) state
-// in registers, so the recurrence needs no cross-thread traffic. Tokens are
-// processed in chunks of GD_TC: a parallel phase prepares unit q/k, decays,
-// beta in LDS; a serial phase runs the recurrence; a parallel phase applies
-// the per-head RMS norm and the sigmoid gate.
-#define GD_TC 8
+// Workgroup = (row, head, block of GD_CW value channels), 256 threads. The
+// (D x Dv) state is kept in registers: GD_PARTS adjacent lanes share one value
+// channel (column) and split its D rows in float4-interleaved order, so a
+// token costs D/GD_PARTS multiply-adds per lane plus two 3-step lane
+// reductions, and no workgroup-wide traffic. Tokens go in chunks of GD_TC: a
+// parallel phase prepares unit q/k, decays and beta in LDS, then the serial
+// recurrence runs on the chunk. Raw read-outs go to an fp32 buffer; the
+// per-head RMS norm and gate need all channels of a head and run in
+// gated_rmsnorm_kernel. State memory layout is (slot, head, Dv, D): a lane's
+// rows are contiguous float4s, a column's rows one contiguous line.
+#define GD_TC 16
+#define GD_THREADS 256
+#define GD_PARTS 8
+#define GD_CW (GD_THREADS / GD_PARTS)
 
-#define GD_MAXTHR 256
-
-template <int DK, typename T, typename TOut>
-__global__ void __launch_bounds__(GD_MAXTHR)
+template <int DK, typename T>
+__global__ void __launch_bounds__(GD_THREADS)
 gated_delta_kernel(const float* __restrict__ qkv, long cstride,
-                                   const T* __restrict__ beta, long bstride,
-                                   const T* __restrict__ a, long astride,
-                                   const T* __restrict__ gate, long gstride,
-                                   const float* __restrict__ dt_bias,
-                                   const float* __restrict__ a_log,
-                                   const float* __restrict__ norm_w, float eps,
-                                   float* __restrict__ state, const int* __restrict__ pos,
-                                   const int* __restrict__ seq, const int* __restrict__ nvalid,
-                                   TOut* __restrict__ out, int S, int H, int G, int D, int Dv) {
-    extern __shared__ float lds[];
-    const int nthr = blockDim.x;
-    const int Dvp = nthr;
-    float* qs = lds;                         // GD_TC * DK
-    float* ks = qs + GD_TC * DK;
-    float* gs = ks + GD_TC * DK;
-    float* os = gs + GD_TC * DK;             // GD_TC * Dvp
-    float* bs = os + GD_TC * Dvp;            // GD_TC
-    const int h = blockIdx.x, b = blockIdx.y;
+                   const T* __restrict__ beta, long bstride,
+                   const T* __restrict__ a, long astride,
+                   const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                   float* __restrict__ state, const int* __restrict__ pos,
+                   const int* __restrict__ seq, const int* __restrict__ nvalid,
+                   float* __restrict__ obuf, int S, int H, int G, int D, int Dv) {
+    constexpr int R = DK / GD_PARTS;         // rows per lane
+    constexpr int F = R / 4;                 // float4s per lane
+    __shared__ __attribute__((aligned(16))) float qs[GD_TC * DK];
+    __shared__ __attribute__((aligned(16))) float ks[GD_TC * DK];
+    __shared__ __attribute__((aligned(16))) float gs[GD_TC * DK];
+    __shared__ float bs[GD_TC];
+    const int h = blockIdx.y, b = blockIdx.z;
     const int slot = seq[b];
     const int n = nvalid[b];
     if (slot < 0 || n <= 0) return;          // uniform over the workgroup
-    const int j = threadIdx.x;
-    const int lane = j & (WAVE - 1), wv = j / WAVE, nw = nthr / WAVE;
-    const bool act = j < Dv;
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1), wv = tid / WAVE;
+    constexpr int NW = GD_THREADS / WAVE;
+    const int part = tid % GD_PARTS;
+    const int col = blockIdx.x * GD_CW + tid / GD_PARTS;
+    const bool act = col < Dv;
     const int g = h / (H / G);
     const int p0 = pos[(long)b * S];
-    float* st = state + ((long)slot * H + h) * D * Dv;
-    float s[DK];
+    float* st = state + (((long)slot * H + h) * Dv + (act ? col : 0)) * D;
+    float s[R];
 #pragma unroll
-    for (int i = 0; i < DK; ++i)
-        s[i] = (act && i < D && p0 > 0) ? st[(long)i * Dv + j] : 0.f;
+    for (int f = 0; f < F; ++f)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = (f * GD_PARTS + part) * 4 + e;
+            s[f * 4 + e] = (act && row < D && p0 > 0) ? st[row] : 0.f;
+        }
     const float neg_rate = -expf(a_log[h]);
     const float qscale = 1.f / sqrtf((float)D);
 
     for (int t0 = 0; t0 < n; t0 += GD_TC) {
         const int tc = min(GD_TC, n - t0);
         const long row0 = (long)b * S + t0;
-        // ---- parallel: unit q / k
-        for (int r = wv; r < 2 * tc; r += nw) {
+        // ---- parallel: unit q / k (one wave per vector)
+        for (int r = wv; r < 2 * tc; r += NW) {
             const int tk = r >> 1, which = r & 1;
             const float* src = qkv + (row0 + tk) * cstride + (which ? G * D : 0) + g * D;
             float ss = 0.f;
@@ -322,7 +346,7 @@ gated_delta_kernel(const float* __restrict__ qkv, long cstride,
             for (int i = lane; i < DK; i += WAVE) dst[i] = i < D ? src[i] * inv : 0.f;
         }
         // ---- parallel: decays and beta
-        for (int idx = j; idx < tc * DK; idx += nthr) {
+        for (int idx = tid; idx < tc * DK; idx += GD_THREADS) {
             const int tk = idx / DK, i = idx % DK;
             float dv = 1.f;
             if (i < D) {
@@ -331,63 +355,85 @@ gated_delta_kernel(const float* __restrict__ qkv, long cstride,
             }
             gs[idx] = dv;
         }
-        if (j < tc) bs[j] = sigmoidf_(ldf<T>(beta + (row0 + j) * bstride + h));
-        float vreg[GD_TC], oreg[GD_TC];
+        if (tid < tc) bs[tid] = sigmoidf_(ldf<T>(beta + (row0 + tid) * bstride + h));
+        float vreg[GD_TC];
 #pragma unroll
         for (int tk = 0; tk < GD_TC; ++tk)
             vreg[tk] = (act && tk < tc)
-                ? qkv[(row0 + tk) * cstride + 2 * G * D + (long)h * Dv + j] : 0.f;
+                ? qkv[(row0 + tk) * cstride + 2 * G * D + (long)h * Dv + col] : 0.f;
         __syncthreads();
         // ---- serial recurrence over the chunk
 #pragma unroll
         for (int tk = 0; tk < GD_TC; ++tk) {
-            oreg[tk] = 0.f;
             if (tk < tc) {
-                const float4* g4 = reinterpret_cast<const float4*>(gs + tk * DK);
-                const float4* k4 = reinterpret_cast<const float4*>(ks + tk * DK);
-                const float4* q4 = reinterpret_cast<const float4*>(qs + tk * DK);
+                const float4* g4 = reinterpret_cast<const float4*>(gs + tk * DK) + part;
+                const float4* k4 = reinterpret_cast<const float4*>(ks + tk * DK) + part;
+                const float4* q4 = reinterpret_cast<const float4*>(qs + tk * DK) + part;
+                float4 kk[F];
                 float dot = 0.f;
 #pragma unroll
-                for (int i = 0; i < DK / 4; ++i) {
-                    const float4 gg = g4[i], kk = k4[i];
-                    s[4 * i] *= gg.x; dot += s[4 * i] * kk.x;
-                    s[4 * i + 1] *= gg.y; dot += s[4 * i + 1] * kk.y;
-                    s[4 * i + 2] *= gg.z; dot += s[4 * i + 2] * kk.z;
-                    s[4 * i + 3] *= gg.w; dot += s[4 * i + 3] * kk.w;
+                for (int f = 0; f < F; ++f) {
+                    const float4 gg = g4[f * GD_PARTS];
+                    kk[f] = k4[f * GD_PARTS];
+                    s[4 * f] *= gg.x; dot += s[4 * f] * kk[f].x;
+                    s[4 * f + 1] *= gg.y; dot += s[4 * f + 1] * kk[f].y;
+                    s[4 * f + 2] *= gg.z; dot += s[4 * f + 2] * kk[f].z;
+                    s[4 * f + 3] *= gg.w; dot += s[4 * f + 3] * kk[f].w;
                 }
+#pragma unroll
+                for (int o = GD_PARTS / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o, WAVE);
                 const float u = bs[tk] * (vreg[tk] - dot);
                 float o = 0.f;
 #pragma unroll
-                for (int i = 0; i < DK / 4; ++i) {
-                    const float4 kk = k4[i], qq = q4[i];
-                    s[4 * i] += kk.x * u; o += s[4 * i] * qq.x;
-                    s[4 * i + 1] += kk.y * u; o += s[4 * i + 1] * qq.y;
-                    s[4 * i + 2] += kk.z * u; o += s[4 * i + 2] * qq.z;
-                    s[4 * i + 3] += kk.w * u; o += s[4 * i + 3] * qq.w;
+                for (int f = 0; f < F; ++f) {
+                    const float4 qq = q4[f * GD_PARTS];
+                    s[4 * f] += kk[f].x * u; o += s[4 * f] * qq.x;
+                    s[4 * f + 1] += kk[f].y * u; o += s[4 * f + 1] * qq.y;
+                    s[4 * f + 2] += kk[f].z * u; o += s[4 * f + 2] * qq.z;
+                    s[4 * f + 3] += kk[f].w * u; o += s[4 * f + 3] * qq.w;
                 }
-                oreg[tk] = o;
-            }
-        }
 #pragma unroll
-        for (int tk = 0; tk < GD_TC; ++tk) os[tk * Dvp + j] = act ? oreg[tk] : 0.f;
-        __syncthreads();
-        // ---- parallel: RMS norm over the value channels, weight, gate
-        for (int tk = wv; tk < tc; tk += nw) {
-            float ss = 0.f;
-            for (int c = lane; c < Dv; c += WAVE) { float o = os[tk * Dvp + c]; ss += o * o; }
-            const float inv = 1.f / sqrtf(wave_sum(ss) / Dv + eps);
-            const T* gp = gate + (row0 + tk) * gstride + (long)h * Dv;
-            TOut* op = out + ((row0 + tk) * H + h) * (long)Dv;
-            for (int c = lane; c < Dv; c += WAVE)
-                stf<TOut>(op + c, os[tk * Dvp + c] * inv * norm_w[c] * sigmoidf_(ldf<T>(gp + c)));
+                for (int x = GD_PARTS / 2; x > 0; x >>= 1) o += __shfl_xor(o, x, WAVE);
+                if (act && part == 0) obuf[((row0 + tk) * H + h) * (long)Dv + col] = o;
+            }
         }
         __syncthreads();
     }
     if (act) {
 #pragma unroll
-        for (int i = 0; i < DK; ++i)
-            if (i < D) st[(long)i * Dv + j] = s[i];
+        for (int f = 0; f < F; ++f)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = (f * GD_PARTS + part) * 4 + e;
+                if (row < D) st[row] = s[f * 4 + e];
+            }
     }
+}
+
+// per-head RMS norm over the value channels, shared weight, sigmoid gate:
+// one wave per (token, head); pad tokens produce zeros
+template <typename T>
+__global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                     long gstride, const float* __restrict__ w, float eps,
+                                     const int* __restrict__ pos, const int* __restrict__ seq,
+                                     T* __restrict__ out, long ntok, int S, int H, int Dv) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const long wid = (long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (wid >= ntok * H) return;
+    const long tok = wid / H;
+    const int h = wid % H;
+    T* op = out + wid * Dv;
+    if (pos[tok] < 0 || seq[tok / S] < 0) {
+        for (int c = lane; c < Dv; c += WAVE) stf<T>(op + c, 0.f);
+        return;
+    }
+    const float* ip = o + wid * Dv;
+    float ss = 0.f;
+    for (int c = lane; c < Dv; c += WAVE) { float v = ip[c]; ss += v * v; }
+    const float inv = 1.f / sqrtf(wave_sum(ss) / Dv + eps);
+    const T* gp = gate + tok * gstride + (long)h * Dv;
+    for (int c = lane; c < Dv; c += WAVE)
+        stf<T>(op + c, ip[c] * inv * w[c] * sigmoidf_(ldf<T>(gp + c)));
 }
 
 // ------------------------------------------------------------- elementwise
@@ -438,8 +484,7 @@ extern "C" {
 int nx_layer_norm(const float* x, const float* w, void* out, int out_bf16, long rows, int C,
                   float eps, hipStream_t st) {
     if (rows <= 0) return 0;
-    const int wpb = 4;
-    dim3 grid((unsigned)((rows + wpb - 1) / wpb)), block(wpb * WAVE);
+    dim3 grid((unsigned)rows), block(LN_THREADS);
     if (out_bf16) layer_norm_kernel<bf16><<<grid, block, 0, st>>>(x, w, (bf16*)out, rows, C, eps);
     else layer_norm_kernel<float><<<grid, block, 0, st>>>(x, w, (float*)out, rows, C, eps);
     return (int)hipGetLastError();
@@ -513,17 +558,15 @@ int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, 
 int nx_gated_delta(const float* qkv, long cstride, const void* beta, long bstride, const void* a,
                    long astride, const void* gate, long gstride, const float* dt_bias,
                    const float* a_log, const float* norm_w, float eps, float* state,
-                   const int* pos, const int* seq, const int* nvalid, void* out, int in_bf16,
-                   int B, int S, int H, int G, int D, int Dv, hipStream_t st) {
+                   const int* pos, const int* seq, const int* nvalid, float* obuf, void* out,
+                   int in_bf16, int B, int S, int H, int G, int D, int Dv, hipStream_t st) {
     if (B <= 0 || S <= 0) return 0;
-    if (D > 256 || Dv > GD_MAXTHR || H % G != 0) return -1;
-    const int nthr = ((Dv + WAVE - 1) / WAVE) * WAVE;
+    if (D > 256 || H % G != 0) return -1;
     const int DK = D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
-    const size_t sh = (size_t)(3 * GD_TC * DK + GD_TC * nthr + GD_TC) * sizeof(float);
-    dim3 grid(H, B), block(nthr);
-#define GD(DKV, T) gated_delta_kernel<DKV, T, T><<<grid, block, sh, st>>>( \
-        qkv, cstride, (const T*)beta, bstride, (const T*)a, astride, (const T*)gate, gstride, \
-        dt_bias, a_log, norm_w, eps, state, pos, seq, nvalid, (T*)out, S, H, G, D, Dv)
+    dim3 grid((Dv + GD_CW - 1) / GD_CW, H, B), block(GD_THREADS);
+#define GD(DKV, T) gated_delta_kernel<DKV, T><<<grid, block, 0, st>>>( \
+        qkv, cstride, (const T*)beta, bstride, (const T*)a, astride, dt_bias, a_log, state, \
+        pos, seq, nvalid, obuf, S, H, G, D, Dv)
 #define GDT(DKV) do { if (in_bf16) GD(DKV, bf16); else GD(DKV, float); } while (0)
     switch (DK) {
         case 32: GDT(32); break;
@@ -533,6 +576,14 @@ int nx_gated_delta(const float* qkv, long cstride, const void* beta, long bstrid
     }
 #undef GDT
 #undef GD
+    int rc = (int)hipGetLastError();
+    if (rc) return rc;
+    const long waves = (long)B * S * H;
+    dim3 g2((unsigned)((waves + 3) / 4)), b2(4 * WAVE);
+    if (in_bf16) gated_rmsnorm_kernel<bf16><<<g2, b2, 0, st>>>(
+        obuf, (const bf16*)gate, gstride, norm_w, eps, pos, seq, (bf16*)out, (long)B * S, S, H, Dv);
+    else gated_rmsnorm_kernel<float><<<g2, b2, 0, st>>>(
+        obuf, (const float*)gate, gstride, norm_w, eps, pos, seq, (float*)out, (long)B * S, S, H, Dv);
     return (int)hipGetLastError();
 }
 

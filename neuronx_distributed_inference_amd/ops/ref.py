@@ -336,7 +336,8 @@ def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps, state,
                      positions, seq_ids, kv_heads, dim, vdim,
                      out_dtype=torch.float32):
     """Delta-rule recurrence with a per-key-channel decay, carried state
-    (slots, H, dim, vdim) fp32. qkv (B,S,2*G*dim + H*vdim) holds the
+    (slots, H, vdim, dim) fp32 (stored transposed: a value channel's key
+    rows are contiguous). qkv (B,S,2*G*dim + H*vdim) holds the
     convolved+activated q|k|v; beta (B,S,H) and a (B,S,H*dim), gate
     (B,S,H*vdim) are pre-activation projections. Per token and head:
       S <- diag(decay) S ; u = beta (v - S^T k) ; S <- S + k u^T ; o = S^T q
@@ -363,13 +364,14 @@ def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps, state,
         n = int(n_valid[b])
         if slot < 0 or n == 0:
             continue
-        St = state[slot].float() if int(p0s[b]) > 0 else torch.zeros_like(state[slot], dtype=torch.float32)
+        St = state[slot].float().transpose(-1, -2) if int(p0s[b]) > 0 else torch.zeros(
+            H, D, Dv, dtype=torch.float32, device=qkv.device)
         for t in range(n):
             St = decay[b, t].unsqueeze(-1) * St
             u = bt[b, t].unsqueeze(-1) * (v[b, t] - torch.einsum("hdv,hd->hv", St, k[b, t]))
             St = St + k[b, t].unsqueeze(-1) * u.unsqueeze(1)
             out[b, t] = torch.einsum("hdv,hd->hv", St, q[b, t])
-        state[slot] = St.to(state.dtype)
+        state[slot] = St.transpose(-1, -2).to(state.dtype)
     out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps) * norm_w.float()
     out = out.reshape(B, S, H * Dv) * torch.sigmoid(gate.float())
     return out.to(out_dtype)

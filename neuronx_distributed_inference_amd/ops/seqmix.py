@@ -225,7 +225,7 @@ def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps: float,
                      state, step: StepLayout, kv_heads: int, dim: int, vdim: int,
                      out_dtype=torch.float32):
     """Gated delta-rule recurrence over the step's tokens, state carried in
-    `state` (slots, H, dim, vdim) fp32; see ref.gated_delta_rule."""
+    `state` (slots, H, vdim, dim) fp32; see ref.gated_delta_rule."""
     if qkv.is_cuda:
         lib = _load()
         B, S = qkv.shape[0], qkv.shape[1]
@@ -233,12 +233,13 @@ def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps: float,
         assert qkv.dtype == torch.float32 and state.dtype == torch.float32
         assert beta.dtype == a.dtype == gate.dtype == out_dtype
         out = torch.empty(B, S, H * vdim, dtype=out_dtype, device=qkv.device)
+        obuf = torch.empty(B, S, H * vdim, dtype=torch.float32, device=qkv.device)
         _check(lib.nx_gated_delta(
             _p(qkv), ctypes.c_long(_rows_view(qkv)), _p(beta),
             ctypes.c_long(_rows_view(beta)), _p(a), ctypes.c_long(_rows_view(a)),
             _p(gate), ctypes.c_long(_rows_view(gate)), _p(_f32(dt_bias)),
             _p(_f32(a_log)), _p(_f32(norm_w)), ctypes.c_float(eps), _p(state),
-            _p(step.positions), _p(step.seq_ids), _p(step.nvalid), _p(out),
+            _p(step.positions), _p(step.seq_ids), _p(step.nvalid), _p(obuf), _p(out),
             _is_bf16(beta), B, S, H, kv_heads, dim, vdim, _stream()),
             "gated_delta_rule")
         return out
