@@ -162,116 +162,253 @@ __global__ void paged_kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc,
 }
 
 // ------------------------------------------------- windowed biased attention
-// One wave per (token, query head). Visible keys of query position i:
-// j in [0, min(keep, lo)) and j in [lo, i], lo = max(0, i-window+1). Lanes
-// take one key each for the scores (online softmax over 64-key tiles), then
-// one value channel each for P.V.
+// Workgroup (4 waves) = ATT_NQ query rows that share one KV head: HPW query
+// heads of the group x QT consecutive tokens of a batch row, so every K/V
+// line fetched serves all of them. The union of the rows' visible keys is
+// [0, min(keep, lo)) + [lo, i_max], lo = max(0, i_min-window+1); each row
+// masks by its own position (j <= i and (i-j < window or j < keep)). Waves
+// take 64-key tiles round-robin: a lane owns one key for the scores (q rows
+// broadcast from LDS, fp32 accumulate, online softmax per row), then the
+// wave's P tile goes through LDS and a lane owns value channels for P.V.
+// The four partial results merge through LDS at the end. One kernel serves
+// prompt portions, decoded tokens and mixed batches.
 #define ATT_WAVES 4
-#define ATT_MAXR 4   // value head size <= 64*ATT_MAXR
+#define ATT_NQ 16
+#define ATT_THREADS (ATT_WAVES * WAVE)
 
-template <typename T, typename TOut>
-__global__ void __launch_bounds__(ATT_WAVES * WAVE)
+template <typename T> struct KVec8 { float v[8]; };
+
+template <typename T> DEV void load8(const T* p, float* v);
+template <> DEV void load8<bf16>(const bf16* p, float* v) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(p);
+    const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        v[2 * e] = __uint_as_float(u[e] << 16);
+        v[2 * e + 1] = __uint_as_float(u[e] & 0xffff0000u);
+    }
+}
+template <> DEV void load8<float>(const float* p, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    const float4 b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+template <typename T, typename TOut, int MAXR>
+__global__ void __launch_bounds__(ATT_THREADS)
 window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ kc,
                    const T* __restrict__ vc, const int* __restrict__ pos,
                    const int* __restrict__ seq,
                    const int* __restrict__ btab, int max_blocks, const float* __restrict__ r1,
                    const float* __restrict__ r2, const T* __restrict__ gate, long gstride,
-                   TOut* __restrict__ out, long ntok, int H, int G, int Dk, int Dv,
-                   int bsz, int S, float scale, int window, int keep) {
-    extern __shared__ float qs[];                      // ATT_WAVES * Dk
-    const int lane = threadIdx.x & (WAVE - 1);
-    const int wv = threadIdx.x / WAVE;
-    const long wid = (long)blockIdx.x * ATT_WAVES + wv;
-    const bool live = wid < ntok * H;
-    const long tok = live ? wid / H : 0;
-    const int h = live ? (int)(wid % H) : 0;
-    const int i = (live && seq[tok / S] >= 0) ? pos[tok] : -1;
-    float* myq = qs + wv * Dk;
-    if (i >= 0) {
-        const T* qp = q + tok * qstride + (long)h * Dk;
-        for (int d = lane; d < Dk; d += WAVE) myq[d] = ldf<T>(qp + d) * scale;
+                   TOut* __restrict__ out, int H, int G, int Dk, int Dv,
+                   int bsz, int S, float scale, int window, int keep, int HPW, int QT,
+                   int chunks) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    const int DkP = (Dk + 7) & ~7;                       // padded q row
+    float* qs = smem;                                    // ATT_NQ * DkP
+    float* ps = qs + ATT_NQ * DkP;                       // ATT_WAVES * 64 * ATT_NQ
+    float* cs = ps + ATT_WAVES * WAVE * ATT_NQ;          // ATT_NQ * Dv + 2 * ATT_NQ
+    __shared__ int rpos[ATT_NQ];
+    __shared__ float ra1[ATT_NQ], ra2[ATT_NQ];
+
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wv = tid / WAVE;
+    const int b = blockIdx.z;
+    const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int t0 = blockIdx.x * QT;
+    const int rep = H / G;
+    if (seq[b] < 0) return;
+    // row table
+    if (tid < ATT_NQ) {
+        const int tq = tid / HPW, hh = chunk * HPW + tid % HPW;
+        int p = -1;
+        if (tq < QT && t0 + tq < S && hh < rep) p = pos[(long)b * S + t0 + tq];
+        rpos[tid] = p;
+        const int h = g * rep + (hh < rep ? hh : 0);
+        ra1[tid] = r1[h];
+        ra2[tid] = r2[h];
     }
     __syncthreads();
-    if (i < 0) return;
-    const int b = tok / S;
-    const int g = h / (H / G);
-    const int* bt = btab + (long)b * max_blocks;
-    const int lo = max(0, i - window + 1);
-    const int nfirst = min(keep, lo);
-    const int n = nfirst + (i - lo + 1);
-    const float a1 = r1[h], a2 = r2[h];
-    float m_run = -INFINITY, l_run = 0.f;
-    float acc[ATT_MAXR];
+    int i_min = 0x7fffffff, i_max = -1;
 #pragma unroll
-    for (int r = 0; r < ATT_MAXR; ++r) acc[r] = 0.f;
-    const long krow = (long)G * Dk, vrow = (long)G * Dv;
+    for (int r = 0; r < ATT_NQ; ++r) {
+        const int p = rpos[r];
+        if (p >= 0) { i_min = min(i_min, p); i_max = max(i_max, p); }
+    }
+    if (i_max < 0) return;                               // uniform
+    // q rows (scaled) into LDS
+    for (int idx = tid; idx < ATT_NQ * DkP; idx += ATT_THREADS) {
+        const int r = idx / DkP, d = idx % DkP;
+        float v = 0.f;
+        if (rpos[r] >= 0 && d < Dk) {
+            const int tq = r / HPW, h = g * rep + chunk * HPW + r % HPW;
+            v = ldf<T>(q + ((long)b * S + t0 + tq) * qstride + (long)h * Dk + d) * scale;
+        }
+        qs[idx] = v;
+    }
+    __syncthreads();
 
-    for (int base = 0; base < n; base += WAVE) {
-        const int m = base + lane;
-        float s = -INFINITY;
-        long slot = 0;
-        if (m < n) {
-            const int j = m < nfirst ? m : lo + (m - nfirst);
-            const int blk = bt[j / bsz];
-            slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);   // unmapped page: row 0, never hit by a live row
-            const T* kp = kc + slot * krow + (long)g * Dk;
-            float dot = 0.f;
-            if constexpr (sizeof(T) == 2) {
-                if ((Dk & 7) == 0) {
-                    for (int d = 0; d < Dk; d += 8) {
-                        const uint4 raw = *reinterpret_cast<const uint4*>(kp + d);
-                        const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+    const int* bt = btab + (long)b * max_blocks;
+    const int lo = max(0, i_min - window + 1);
+    const int nfirst = min(keep, lo);
+    const int n = nfirst + (i_max - lo + 1);
+    const int ntiles = (n + WAVE - 1) / WAVE;
+    const int rounds = (ntiles + ATT_WAVES - 1) / ATT_WAVES;
+    const long krow = (long)G * Dk, vrow = (long)G * Dv;
+    float m_run[ATT_NQ], l_run[ATT_NQ], acc[ATT_NQ][MAXR];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            dot += __uint_as_float(u[e] << 16) * myq[d + 2 * e];
-                            dot += __uint_as_float(u[e] & 0xffff0000u) * myq[d + 2 * e + 1];
-                        }
+    for (int r = 0; r < ATT_NQ; ++r) {
+        m_run[r] = -INFINITY; l_run[r] = 0.f;
+#pragma unroll
+        for (int c = 0; c < MAXR; ++c) acc[r][c] = 0.f;
+    }
+    float* myp = ps + wv * WAVE * ATT_NQ;
+
+    for (int rd = 0; rd < rounds; ++rd) {
+        const int base = (rd * ATT_WAVES + wv) * WAVE;
+        const int m = base + lane;
+        const bool kvalid = m < n;
+        int j = 0;
+        long slot = 0;
+        float sc[ATT_NQ];
+#pragma unroll
+        for (int r = 0; r < ATT_NQ; ++r) sc[r] = 0.f;
+        if (base < n) {                                  // wave-uniform
+            if (kvalid) {
+                j = m < nfirst ? m : lo + (m - nfirst);
+                const int blk = bt[j / bsz];
+                slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
+            }
+            const T* kp = kc + slot * krow + (long)g * Dk;
+            if ((Dk & 7) == 0) {
+                for (int d = 0; d < Dk; d += 8) {
+                    float kv[8];
+                    load8<T>(kp + d, kv);
+#pragma unroll
+                    for (int r = 0; r < ATT_NQ; ++r) {
+                        if (rpos[r] < 0) continue;       // uniform
+                        const float4 qa = *reinterpret_cast<const float4*>(qs + r * DkP + d);
+                        const float4 qb = *reinterpret_cast<const float4*>(qs + r * DkP + d + 4);
+                        sc[r] += kv[0] * qa.x + kv[1] * qa.y + kv[2] * qa.z + kv[3] * qa.w +
+                                 kv[4] * qb.x + kv[5] * qb.y + kv[6] * qb.z + kv[7] * qb.w;
                     }
-                } else {
-                    for (int d = 0; d < Dk; ++d) dot += ldf<T>(kp + d) * myq[d];
                 }
             } else {
-                if ((Dk & 3) == 0) {
-                    for (int d = 0; d < Dk; d += 4) {
-                        const float4 kv = *reinterpret_cast<const float4*>(kp + d);
-                        dot += kv.x * myq[d] + kv.y * myq[d + 1] + kv.z * myq[d + 2] +
-                               kv.w * myq[d + 3];
-                    }
-                } else {
-                    for (int d = 0; d < Dk; ++d) dot += ldf<T>(kp + d) * myq[d];
+                for (int d = 0; d < Dk; ++d) {
+                    const float kvs = ldf<T>(kp + d);
+#pragma unroll
+                    for (int r = 0; r < ATT_NQ; ++r) sc[r] += kvs * qs[r * DkP + d];
                 }
             }
-            s = dot - a1 * log1pf(a2 * (float)(i - j));
+            // bias, mask, online softmax per row
+#pragma unroll
+            for (int r = 0; r < ATT_NQ; ++r) {
+                const int i = rpos[r];
+                if (i < 0) continue;                     // uniform
+                const int dist = i - j;
+                const bool vis = kvalid && dist >= 0 && (dist < window || j < keep);
+                float sv = -INFINITY;
+                if (vis) {
+                    const float x = ra2[r] * (float)dist;
+                    const float lg = sizeof(T) == 4 ? log1pf(x) : __logf(1.f + x);
+                    sv = sc[r] - ra1[r] * lg;
+                }
+                const float m_new = fmaxf(m_run[r], wave_max(sv));
+                float p = 0.f, corr = 1.f;
+                if (m_new > -INFINITY) {
+                    p = vis ? expf(sv - m_new) : 0.f;
+                    corr = expf(m_run[r] - m_new);
+                }
+                l_run[r] = l_run[r] * corr + wave_sum(p);
+                m_run[r] = m_new;
+#pragma unroll
+                for (int c = 0; c < MAXR; ++c) acc[r][c] *= corr;
+                sc[r] = p;
+            }
+#pragma unroll
+            for (int r = 0; r < ATT_NQ; ++r) myp[lane * ATT_NQ + r] = sc[r];
         }
-        const float m_new = fmaxf(m_run, wave_max(s));
-        const float p = (m < n) ? expf(s - m_new) : 0.f;
-        const float corr = expf(m_run - m_new);        // 0 on the first tile
-        l_run = l_run * corr + wave_sum(p);
-        m_run = m_new;
+        __syncthreads();
+        if (base < n) {
+            const int cnt = min(WAVE, n - base);
+            const int sl = (int)slot;
+            for (int mm = 0; mm < cnt; ++mm) {
+                const long sj = __shfl(sl, mm, WAVE);
+                const T* vp = vc + sj * vrow + (long)g * Dv;
+                float vv[MAXR];
 #pragma unroll
-        for (int r = 0; r < ATT_MAXR; ++r) acc[r] *= corr;
-        const int cnt = min(WAVE, n - base);
-        for (int mm = 0; mm < cnt; ++mm) {
-            const float pj = __shfl(p, mm, WAVE);
-            const long sj = __shfl((int)slot, mm, WAVE);
-            const T* vp = vc + sj * vrow + (long)g * Dv;
+                for (int c = 0; c < MAXR; ++c) {
+                    const int d = lane + c * WAVE;
+                    vv[c] = d < Dv ? ldf<T>(vp + d) : 0.f;
+                }
+                const float4* p4 = reinterpret_cast<const float4*>(myp + mm * ATT_NQ);
 #pragma unroll
-            for (int r = 0; r < ATT_MAXR; ++r) {
-                const int d = lane + r * WAVE;
-                if (d < Dv) acc[r] += pj * ldf<T>(vp + d);
+                for (int r4 = 0; r4 < ATT_NQ / 4; ++r4) {
+                    const float4 pp = p4[r4];
+#pragma unroll
+                    for (int c = 0; c < MAXR; ++c) {
+                        acc[4 * r4][c] += pp.x * vv[c];
+                        acc[4 * r4 + 1][c] += pp.y * vv[c];
+                        acc[4 * r4 + 2][c] += pp.z * vv[c];
+                        acc[4 * r4 + 3][c] += pp.w * vv[c];
+                    }
+                }
             }
         }
+        __syncthreads();
     }
-    const float inv = 1.f / l_run;
-    TOut* op = out + (tok * H + h) * (long)Dv;
-    const T* gp = gate ? gate + tok * gstride + (long)h * Dv : nullptr;
+    // merge the waves' partial softmaxes: wave 3 -> 2 -> 1 -> 0 through LDS
+    float* cm = cs + ATT_NQ * Dv;
+    float* cl = cm + ATT_NQ;
+    for (int src = ATT_WAVES - 1; src >= 1; --src) {
+        if (wv == src) {
 #pragma unroll
-    for (int r = 0; r < ATT_MAXR; ++r) {
-        const int d = lane + r * WAVE;
-        if (d < Dv) {
-            float o = acc[r] * inv;
-            if (gp) o *= sigmoidf_(ldf<T>(gp + d));
-            stf<TOut>(op + d, o);
+            for (int r = 0; r < ATT_NQ; ++r) {
+                if (lane == 0) { cm[r] = m_run[r]; cl[r] = l_run[r]; }
+#pragma unroll
+                for (int c = 0; c < MAXR; ++c) {
+                    const int d = lane + c * WAVE;
+                    if (d < Dv) cs[r * Dv + d] = acc[r][c];
+                }
+            }
+        }
+        __syncthreads();
+        if (wv == src - 1) {
+#pragma unroll
+            for (int r = 0; r < ATT_NQ; ++r) {
+                const float mo = cm[r], lo2 = cl[r];
+                const float m_new = fmaxf(m_run[r], mo);
+                float ca = 1.f, cb = 0.f;
+                if (m_new > -INFINITY) { ca = expf(m_run[r] - m_new); cb = expf(mo - m_new); }
+                l_run[r] = l_run[r] * ca + lo2 * cb;
+                m_run[r] = m_new;
+#pragma unroll
+                for (int c = 0; c < MAXR; ++c) {
+                    const int d = lane + c * WAVE;
+                    if (d < Dv) acc[r][c] = acc[r][c] * ca + cs[r * Dv + d] * cb;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (wv != 0) return;
+#pragma unroll
+    for (int r = 0; r < ATT_NQ; ++r) {
+        if (rpos[r] < 0) continue;
+        const int tq = r / HPW, h = g * rep + chunk * HPW + r % HPW;
+        const long tok = (long)b * S + t0 + tq;
+        const float inv = 1.f / l_run[r];
+        TOut* op = out + (tok * H + h) * (long)Dv;
+        const T* gp = gate ? gate + tok * gstride + (long)h * Dv : nullptr;
+#pragma unroll
+        for (int c = 0; c < MAXR; ++c) {
+            const int d = lane + c * WAVE;
+            if (d < Dv) {
+                float o = acc[r][c] * inv;
+                if (gp) o *= sigmoidf_(ldf<T>(gp + d));
+                stf<TOut>(op + d, o);
+            }
         }
     }
 }
@@ -534,23 +671,31 @@ int nx_paged_kv_write(void* kc, void* vc, const void* k, long kstride, const voi
 }
 
 int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, const int* pos,
-                   const int* seq, const int* btab, int max_blocks, const float* r1, const float* r2,
-                   const void* gate, long gstride, void* out, int io_bf16, int out_bf16,
-                   int B, int S, int H, int G, int Dk, int Dv, int bsz, float scale, int window,
-                   int keep, hipStream_t st) {
-    const long ntok = (long)B * S;
-    if (ntok <= 0) return 0;
-    if (Dv > WAVE * ATT_MAXR || H % G != 0) return -1;
-    const long waves = ntok * H;
-    dim3 grid((unsigned)((waves + ATT_WAVES - 1) / ATT_WAVES)), block(ATT_WAVES * WAVE);
-    const size_t sh = (size_t)ATT_WAVES * Dk * sizeof(float);
-#define WA(T, TO) window_attn_kernel<T, TO><<<grid, block, sh, st>>>( \
+                   const int* seq, const int* btab, int max_blocks, const float* r1,
+                   const float* r2, const void* gate, long gstride, void* out, int io_bf16,
+                   int out_bf16, int B, int S, int H, int G, int Dk, int Dv, int bsz,
+                   float scale, int window, int keep, hipStream_t st) {
+    if ((long)B * S <= 0) return 0;
+    if (Dv > WAVE * 4 || H % G != 0) return -1;
+    const int rep = H / G;
+    const int HPW = rep < ATT_NQ ? rep : ATT_NQ;          // query heads per workgroup
+    const int QT = ATT_NQ / HPW;                          // tokens per workgroup
+    const int chunks = (rep + HPW - 1) / HPW;
+    const int DkP = (Dk + 7) & ~7;
+    dim3 grid((S + QT - 1) / QT, G * chunks, B), block(ATT_THREADS);
+    const size_t sh = (size_t)(ATT_NQ * DkP + ATT_WAVES * WAVE * ATT_NQ + ATT_NQ * Dv +
+                               2 * ATT_NQ) * sizeof(float);
+    if (sh > 60 * 1024) return -3;
+#define WA(T, TO, MR) window_attn_kernel<T, TO, MR><<<grid, block, sh, st>>>( \
         (const T*)q, qstride, (const T*)kc, (const T*)vc, pos, seq, btab, max_blocks, r1, r2, \
-        (const T*)gate, gstride, (TO*)out, ntok, H, G, Dk, Dv, bsz, S, scale, window, keep)
-    if (io_bf16 && out_bf16) WA(bf16, bf16);
-    else if (io_bf16) WA(bf16, float);
+        (const T*)gate, gstride, (TO*)out, H, G, Dk, Dv, bsz, S, scale, window, keep, HPW, QT, \
+        chunks)
+#define WAM(T, TO) do { if (Dv <= 2 * WAVE) WA(T, TO, 2); else WA(T, TO, 4); } while (0)
+    if (io_bf16 && out_bf16) WAM(bf16, bf16);
+    else if (io_bf16) WAM(bf16, float);
     else if (out_bf16) return -2;
-    else WA(float, float);
+    else WAM(float, float);
+#undef WAM
 #undef WA
     return (int)hipGetLastError();
 }
