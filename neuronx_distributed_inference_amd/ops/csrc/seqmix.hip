@@ -172,9 +172,10 @@ __global__ void paged_kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc,
 // wave's P tile goes through LDS and a lane owns value channels for P.V.
 // The four partial results merge through LDS at the end. One kernel serves
 // prompt portions, decoded tokens and mixed batches.
-#define ATT_WAVES 4
-#define ATT_NQ 16
-#define ATT_THREADS (ATT_WAVES * WAVE)
+// Two shapes: (NQ=16 rows, 4 waves) for steps with prompt portions, and
+// (NQ=4 rows, 16 waves) for pure decode steps, where one token's few heads
+// leave the key range as the only parallelism.
+#define ATT_NQ_MAX 16
 
 template <typename T> struct KVec8 { float v[8]; };
 
@@ -195,8 +196,8 @@ template <> DEV void load8<float>(const float* p, float* v) {
     v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
 }
 
-template <typename T, typename TOut, int MAXR>
-__global__ void __launch_bounds__(ATT_THREADS)
+template <typename T, typename TOut, int MAXR, int ATT_NQ, int ATT_WAVES>
+__global__ void __launch_bounds__(ATT_WAVES * WAVE)
 window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ kc,
                    const T* __restrict__ vc, const int* __restrict__ pos,
                    const int* __restrict__ seq,
@@ -209,9 +210,10 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
     const int DkP = (Dk + 7) & ~7;                       // padded q row
     float* qs = smem;                                    // ATT_NQ * DkP
     float* ps = qs + ATT_NQ * DkP;                       // ATT_WAVES * 64 * ATT_NQ
-    float* cs = ps + ATT_WAVES * WAVE * ATT_NQ;          // ATT_NQ * Dv + 2 * ATT_NQ
-    __shared__ int rpos[ATT_NQ];
-    __shared__ float ra1[ATT_NQ], ra2[ATT_NQ];
+    float* cs = ps;                                      // merge area reuses the P tiles
+    constexpr int ATT_THREADS = ATT_WAVES * WAVE;
+    __shared__ int rpos[ATT_NQ_MAX];
+    __shared__ float ra1[ATT_NQ_MAX], ra2[ATT_NQ_MAX];
 
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wv = tid / WAVE;
     const int b = blockIdx.z;
@@ -358,23 +360,24 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
         }
         __syncthreads();
     }
-    // merge the waves' partial softmaxes: wave 3 -> 2 -> 1 -> 0 through LDS
-    float* cm = cs + ATT_NQ * Dv;
-    float* cl = cm + ATT_NQ;
-    for (int src = ATT_WAVES - 1; src >= 1; --src) {
-        if (wv == src) {
+    // merge the waves' partial softmaxes pairwise (tree) through LDS
+    for (int step = 1; step < ATT_WAVES; step <<= 1) {
+        float* slot_acc = cs + (wv / (2 * step)) * ATT_NQ * (Dv + 2);
+        float* cm = slot_acc + ATT_NQ * Dv;
+        float* cl = cm + ATT_NQ;
+        if (wv % (2 * step) == step) {
 #pragma unroll
             for (int r = 0; r < ATT_NQ; ++r) {
                 if (lane == 0) { cm[r] = m_run[r]; cl[r] = l_run[r]; }
 #pragma unroll
                 for (int c = 0; c < MAXR; ++c) {
                     const int d = lane + c * WAVE;
-                    if (d < Dv) cs[r * Dv + d] = acc[r][c];
+                    if (d < Dv) slot_acc[r * Dv + d] = acc[r][c];
                 }
             }
         }
         __syncthreads();
-        if (wv == src - 1) {
+        if (wv % (2 * step) == 0 && wv + step < ATT_WAVES) {
 #pragma unroll
             for (int r = 0; r < ATT_NQ; ++r) {
                 const float mo = cm[r], lo2 = cl[r];
@@ -386,7 +389,7 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
 #pragma unroll
                 for (int c = 0; c < MAXR; ++c) {
                     const int d = lane + c * WAVE;
-                    if (d < Dv) acc[r][c] = acc[r][c] * ca + cs[r * Dv + d] * cb;
+                    if (d < Dv) acc[r][c] = acc[r][c] * ca + slot_acc[r * Dv + d] * cb;
                 }
             }
         }
@@ -414,45 +417,87 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
 }
 
 // ------------------------------------------------------- gated delta rule
-// Workgroup = (row, head, block of GD_CW value channels), 256 threads. The
-// (D x Dv) state is kept in registers: GD_PARTS adjacent lanes share one value
-// channel (column) and split its D rows in float4-interleaved order, so a
-// token costs D/GD_PARTS multiply-adds per lane plus two 3-step lane
-// reductions, and no workgroup-wide traffic. Tokens go in chunks of GD_TC: a
-// parallel phase prepares unit q/k, decays and beta in LDS, then the serial
-// recurrence runs on the chunk. Raw read-outs go to an fp32 buffer; the
-// per-head RMS norm and gate need all channels of a head and run in
-// gated_rmsnorm_kernel. State memory layout is (slot, head, Dv, D): a lane's
-// rows are contiguous float4s, a column's rows one contiguous line.
-#define GD_TC 16
+// Three kernels per step.
+// (1) delta_prep_kernel, fully parallel over tokens: unit q and k per KV head
+//     (q also scaled by D^-1/2), decay exp(-exp(A_log) softplus(a + dt_bias))
+//     per head and key channel, beta = sigmoid(.), all fp32, into one row per
+//     token: [q (G*D) | k (G*D) | decay (H*D) | beta (H)], stride PS.
+// (2) gated_delta_kernel, the serial scan. Workgroup = (row, head, block of
+//     GD_CW value channels), 256 threads. The (D x Dv) state is kept in
+//     registers: GD_PARTS adjacent lanes share one value channel (column) and
+//     split its D rows in float4-interleaved order, so a token costs
+//     D/GD_PARTS multiply-adds per lane plus two 3-step lane reductions and no
+//     workgroup-wide traffic. Tokens go in chunks of TC through LDS; the next
+//     chunk's rows are fetched into registers while the current one is
+//     scanned. State memory layout is (slot, head, Dv, D): a lane's rows are
+//     contiguous float4s, a column's rows one contiguous line.
+// (3) gated_rmsnorm_kernel: per-head RMS norm, weight and sigmoid gate (needs
+//     all value channels of a head, which (2) spreads over workgroups).
 #define GD_THREADS 256
 #define GD_PARTS 8
 #define GD_CW (GD_THREADS / GD_PARTS)
 
-template <int DK, typename T>
+template <typename T>
+__global__ void delta_prep_kernel(const float* __restrict__ qkv, long cstride,
+                                  const T* __restrict__ beta, long bstride,
+                                  const T* __restrict__ a, long astride,
+                                  const float* __restrict__ dt_bias,
+                                  const float* __restrict__ a_log, const int* __restrict__ pos,
+                                  const int* __restrict__ seq, float* __restrict__ prep, long PS,
+                                  long ntok, int S, int H, int G, int D) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int units = 2 * G + H;
+    const long wid = (long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (wid >= ntok * units) return;
+    const long tok = wid / units;
+    const int u = wid % units;
+    if (pos[tok] < 0 || seq[tok / S] < 0) return;
+    float* pr = prep + tok * PS;
+    if (u < 2 * G) {
+        const float* src = qkv + tok * cstride + (long)u * D;      // q heads then k heads
+        float ss = 0.f;
+        for (int i = lane; i < D; i += WAVE) { float x = src[i]; ss += x * x; }
+        float inv = 1.f / sqrtf(wave_sum(ss) + 1e-6f);
+        if (u < G) inv *= 1.f / sqrtf((float)D);
+        for (int i = lane; i < D; i += WAVE) pr[(long)u * D + i] = src[i] * inv;
+    } else {
+        const int h = u - 2 * G;
+        const float neg_rate = -expf(a_log[h]);
+        const T* ap = a + tok * astride + (long)h * D;
+        for (int i = lane; i < D; i += WAVE)
+            pr[(long)(2 * G + h) * D + i] =
+                expf(neg_rate * softplusf_(ldf<T>(ap + i) + dt_bias[h * D + i]));
+        if (lane == 0)
+            pr[(long)(2 * G + H) * D + h] = sigmoidf_(ldf<T>(beta + tok * bstride + h));
+    }
+}
+
+template <int DK, int TC>
 __global__ void __launch_bounds__(GD_THREADS)
-gated_delta_kernel(const float* __restrict__ qkv, long cstride,
-                   const T* __restrict__ beta, long bstride,
-                   const T* __restrict__ a, long astride,
-                   const float* __restrict__ dt_bias, const float* __restrict__ a_log,
-                   float* __restrict__ state, const int* __restrict__ pos,
+gated_delta_kernel(const float* __restrict__ qkv, long cstride, const float* __restrict__ prep,
+                   long PS, float* __restrict__ state, const int* __restrict__ pos,
                    const int* __restrict__ seq, const int* __restrict__ nvalid,
                    float* __restrict__ obuf, int S, int H, int G, int D, int Dv) {
     constexpr int R = DK / GD_PARTS;         // rows per lane
     constexpr int F = R / 4;                 // float4s per lane
-    __shared__ __attribute__((aligned(16))) float qs[GD_TC * DK];
-    __shared__ __attribute__((aligned(16))) float ks[GD_TC * DK];
-    __shared__ __attribute__((aligned(16))) float gs[GD_TC * DK];
-    __shared__ float bs[GD_TC];
+    constexpr int NQKG = 3 * TC * DK;        // LDS floats per chunk: q | k | decay
+    constexpr int NE = NQKG + TC * GD_CW + TC;   // ... | v (TC x GD_CW) | beta (TC)
+    constexpr int PER = (NE + GD_THREADS - 1) / GD_THREADS;
+    __shared__ __attribute__((aligned(16))) float buf[PER * GD_THREADS];
+    const float* qs = buf;
+    const float* ks = buf + TC * DK;
+    const float* gs = buf + 2 * TC * DK;
+    const float* vs = buf + NQKG;
+    const float* bs = vs + TC * GD_CW;
     const int h = blockIdx.y, b = blockIdx.z;
     const int slot = seq[b];
     const int n = nvalid[b];
     if (slot < 0 || n <= 0) return;          // uniform over the workgroup
     const int tid = threadIdx.x;
-    const int lane = tid & (WAVE - 1), wv = tid / WAVE;
-    constexpr int NW = GD_THREADS / WAVE;
     const int part = tid % GD_PARTS;
-    const int col = blockIdx.x * GD_CW + tid / GD_PARTS;
+    const int cl = tid / GD_PARTS;
+    const int col0 = blockIdx.x * GD_CW;
+    const int col = col0 + cl;
     const bool act = col < Dv;
     const int g = h / (H / G);
     const int p0 = pos[(long)b * S];
@@ -465,77 +510,76 @@ gated_delta_kernel(const float* __restrict__ qkv, long cstride,
             const int row = (f * GD_PARTS + part) * 4 + e;
             s[f * 4 + e] = (act && row < D && p0 > 0) ? st[row] : 0.f;
         }
-    const float neg_rate = -expf(a_log[h]);
-    const float qscale = 1.f / sqrtf((float)D);
+    const long off_q = (long)g * D, off_k = (long)(G + g) * D, off_g = (long)(2 * G + h) * D;
+    const long off_b = (long)(2 * G + H) * D + h;
+    const long off_v = 2L * G * D + (long)h * Dv + col0;
 
-    for (int t0 = 0; t0 < n; t0 += GD_TC) {
-        const int tc = min(GD_TC, n - t0);
+    float pre[PER];
+    // chunk at t0 -> registers (loads are issued, not waited for)
+#define GD_FETCH(T0)                                                                      \
+    {                                                                                     \
+        const int ftc = min(TC, n - (T0));                                                \
+        const long frow = (long)b * S + (T0);                                             \
+        _Pragma("unroll") for (int x = 0; x < PER; ++x) {                                 \
+            const int idx = tid + x * GD_THREADS;                                         \
+            float v = 0.f;                                                                \
+            if (idx < NQKG) {                                                             \
+                const int which = idx / (TC * DK), rem = idx % (TC * DK);                 \
+                const int tk = rem / DK, i = rem % DK;                                    \
+                if (tk < ftc && i < D)                                                    \
+                    v = prep[(frow + tk) * PS + (which == 0 ? off_q : which == 1 ? off_k : off_g) + i]; \
+            } else if (idx < NQKG + TC * GD_CW) {                                         \
+                const int tk = (idx - NQKG) / GD_CW, c = (idx - NQKG) % GD_CW;            \
+                if (tk < ftc && col0 + c < Dv) v = qkv[(frow + tk) * cstride + off_v + c]; \
+            } else if (idx < NE) {                                                        \
+                const int tk = idx - NQKG - TC * GD_CW;                                   \
+                if (tk < ftc) v = prep[(frow + tk) * PS + off_b];                         \
+            }                                                                             \
+            pre[x] = v;                                                                   \
+        }                                                                                 \
+    }
+    GD_FETCH(0)
+    for (int t0 = 0; t0 < n; t0 += TC) {
+        const int tc = min(TC, n - t0);
         const long row0 = (long)b * S + t0;
-        // ---- parallel: unit q / k (one wave per vector)
-        for (int r = wv; r < 2 * tc; r += NW) {
-            const int tk = r >> 1, which = r & 1;
-            const float* src = qkv + (row0 + tk) * cstride + (which ? G * D : 0) + g * D;
-            float ss = 0.f;
-            for (int i = lane; i < D; i += WAVE) { float x = src[i]; ss += x * x; }
-            float inv = 1.f / sqrtf(wave_sum(ss) + 1e-6f);
-            if (!which) inv *= qscale;
-            float* dst = (which ? ks : qs) + tk * DK;
-            for (int i = lane; i < DK; i += WAVE) dst[i] = i < D ? src[i] * inv : 0.f;
-        }
-        // ---- parallel: decays and beta
-        for (int idx = tid; idx < tc * DK; idx += GD_THREADS) {
-            const int tk = idx / DK, i = idx % DK;
-            float dv = 1.f;
-            if (i < D) {
-                const float z = ldf<T>(a + (row0 + tk) * astride + h * D + i) + dt_bias[h * D + i];
-                dv = expf(neg_rate * softplusf_(z));
-            }
-            gs[idx] = dv;
-        }
-        if (tid < tc) bs[tid] = sigmoidf_(ldf<T>(beta + (row0 + tid) * bstride + h));
-        float vreg[GD_TC];
 #pragma unroll
-        for (int tk = 0; tk < GD_TC; ++tk)
-            vreg[tk] = (act && tk < tc)
-                ? qkv[(row0 + tk) * cstride + 2 * G * D + (long)h * Dv + col] : 0.f;
+        for (int x = 0; x < PER; ++x) buf[tid + x * GD_THREADS] = pre[x];
         __syncthreads();
-        // ---- serial recurrence over the chunk
+        if (t0 + TC < n) GD_FETCH(t0 + TC)   // in flight during the scan below
+        for (int tk = 0; tk < tc; ++tk) {
+            const float4* g4 = reinterpret_cast<const float4*>(gs + tk * DK) + part;
+            const float4* k4 = reinterpret_cast<const float4*>(ks + tk * DK) + part;
+            const float4* q4 = reinterpret_cast<const float4*>(qs + tk * DK) + part;
+            float4 kk[F];
+            float dot = 0.f;
 #pragma unroll
-        for (int tk = 0; tk < GD_TC; ++tk) {
-            if (tk < tc) {
-                const float4* g4 = reinterpret_cast<const float4*>(gs + tk * DK) + part;
-                const float4* k4 = reinterpret_cast<const float4*>(ks + tk * DK) + part;
-                const float4* q4 = reinterpret_cast<const float4*>(qs + tk * DK) + part;
-                float4 kk[F];
-                float dot = 0.f;
-#pragma unroll
-                for (int f = 0; f < F; ++f) {
-                    const float4 gg = g4[f * GD_PARTS];
-                    kk[f] = k4[f * GD_PARTS];
-                    s[4 * f] *= gg.x; dot += s[4 * f] * kk[f].x;
-                    s[4 * f + 1] *= gg.y; dot += s[4 * f + 1] * kk[f].y;
-                    s[4 * f + 2] *= gg.z; dot += s[4 * f + 2] * kk[f].z;
-                    s[4 * f + 3] *= gg.w; dot += s[4 * f + 3] * kk[f].w;
-                }
-#pragma unroll
-                for (int o = GD_PARTS / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o, WAVE);
-                const float u = bs[tk] * (vreg[tk] - dot);
-                float o = 0.f;
-#pragma unroll
-                for (int f = 0; f < F; ++f) {
-                    const float4 qq = q4[f * GD_PARTS];
-                    s[4 * f] += kk[f].x * u; o += s[4 * f] * qq.x;
-                    s[4 * f + 1] += kk[f].y * u; o += s[4 * f + 1] * qq.y;
-                    s[4 * f + 2] += kk[f].z * u; o += s[4 * f + 2] * qq.z;
-                    s[4 * f + 3] += kk[f].w * u; o += s[4 * f + 3] * qq.w;
-                }
-#pragma unroll
-                for (int x = GD_PARTS / 2; x > 0; x >>= 1) o += __shfl_xor(o, x, WAVE);
-                if (act && part == 0) obuf[((row0 + tk) * H + h) * (long)Dv + col] = o;
+            for (int f = 0; f < F; ++f) {
+                const float4 gg = g4[f * GD_PARTS];
+                kk[f] = k4[f * GD_PARTS];
+                s[4 * f] *= gg.x; dot += s[4 * f] * kk[f].x;
+                s[4 * f + 1] *= gg.y; dot += s[4 * f + 1] * kk[f].y;
+                s[4 * f + 2] *= gg.z; dot += s[4 * f + 2] * kk[f].z;
+                s[4 * f + 3] *= gg.w; dot += s[4 * f + 3] * kk[f].w;
             }
+#pragma unroll
+            for (int o = GD_PARTS / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o, WAVE);
+            const float u = bs[tk] * (vs[tk * GD_CW + cl] - dot);
+            float o = 0.f;
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                const float4 qq = q4[f * GD_PARTS];
+                s[4 * f] += kk[f].x * u; o += s[4 * f] * qq.x;
+                s[4 * f + 1] += kk[f].y * u; o += s[4 * f + 1] * qq.y;
+                s[4 * f + 2] += kk[f].z * u; o += s[4 * f + 2] * qq.z;
+                s[4 * f + 3] += kk[f].w * u; o += s[4 * f + 3] * qq.w;
+            }
+#pragma unroll
+            for (int x = GD_PARTS / 2; x > 0; x >>= 1) o += __shfl_xor(o, x, WAVE);
+            if (act && part == 0) obuf[((row0 + tk) * H + h) * (long)Dv + col] = o;
         }
         __syncthreads();
     }
+#undef GD_FETCH
     if (act) {
 #pragma unroll
         for (int f = 0; f < F; ++f)
@@ -677,25 +721,29 @@ int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, 
                    float scale, int window, int keep, hipStream_t st) {
     if ((long)B * S <= 0) return 0;
     if (Dv > WAVE * 4 || H % G != 0) return -1;
+    if (!io_bf16 && out_bf16) return -2;
+    const bool dec = S == 1;                              // pure decode step
+    const int NQ = dec ? 4 : 16, NW = dec ? 16 : 4;
     const int rep = H / G;
-    const int HPW = rep < ATT_NQ ? rep : ATT_NQ;          // query heads per workgroup
-    const int QT = ATT_NQ / HPW;                          // tokens per workgroup
+    const int HPW = rep < NQ ? rep : NQ;                  // query heads per workgroup
+    const int QT = NQ / HPW;                              // tokens per workgroup
     const int chunks = (rep + HPW - 1) / HPW;
     const int DkP = (Dk + 7) & ~7;
-    dim3 grid((S + QT - 1) / QT, G * chunks, B), block(ATT_THREADS);
-    const size_t sh = (size_t)(ATT_NQ * DkP + ATT_WAVES * WAVE * ATT_NQ + ATT_NQ * Dv +
-                               2 * ATT_NQ) * sizeof(float);
+    dim3 grid((S + QT - 1) / QT, G * chunks, B), block(NW * WAVE);
+    const long ptile = (long)NW * WAVE * NQ, marea = (long)(NW / 2) * NQ * (Dv + 2);
+    const size_t sh = (size_t)(NQ * DkP + (ptile > marea ? ptile : marea)) * sizeof(float);
     if (sh > 60 * 1024) return -3;
-#define WA(T, TO, MR) window_attn_kernel<T, TO, MR><<<grid, block, sh, st>>>( \
+#define WA(T, TO, MR, Q, W) window_attn_kernel<T, TO, MR, Q, W><<<grid, block, sh, st>>>( \
         (const T*)q, qstride, (const T*)kc, (const T*)vc, pos, seq, btab, max_blocks, r1, r2, \
         (const T*)gate, gstride, (TO*)out, H, G, Dk, Dv, bsz, S, scale, window, keep, HPW, QT, \
         chunks)
-#define WAM(T, TO) do { if (Dv <= 2 * WAVE) WA(T, TO, 2); else WA(T, TO, 4); } while (0)
+#define WAS(T, TO, MR) do { if (dec) WA(T, TO, MR, 4, 16); else WA(T, TO, MR, 16, 4); } while (0)
+#define WAM(T, TO) do { if (Dv <= 2 * WAVE) WAS(T, TO, 2); else WAS(T, TO, 4); } while (0)
     if (io_bf16 && out_bf16) WAM(bf16, bf16);
     else if (io_bf16) WAM(bf16, float);
-    else if (out_bf16) return -2;
     else WAM(float, float);
 #undef WAM
+#undef WAS
 #undef WA
     return (int)hipGetLastError();
 }
@@ -703,32 +751,40 @@ int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, 
 int nx_gated_delta(const float* qkv, long cstride, const void* beta, long bstride, const void* a,
                    long astride, const void* gate, long gstride, const float* dt_bias,
                    const float* a_log, const float* norm_w, float eps, float* state,
-                   const int* pos, const int* seq, const int* nvalid, float* obuf, void* out,
-                   int in_bf16, int B, int S, int H, int G, int D, int Dv, hipStream_t st) {
+                   const int* pos, const int* seq, const int* nvalid, float* prep, long PS,
+                   float* obuf, void* out, int in_bf16, int B, int S, int H, int G, int D,
+                   int Dv, hipStream_t st) {
     if (B <= 0 || S <= 0) return 0;
-    if (D > 256 || H % G != 0) return -1;
-    const int DK = D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
-    dim3 grid((Dv + GD_CW - 1) / GD_CW, H, B), block(GD_THREADS);
-#define GD(DKV, T) gated_delta_kernel<DKV, T><<<grid, block, 0, st>>>( \
-        qkv, cstride, (const T*)beta, bstride, (const T*)a, astride, dt_bias, a_log, state, \
-        pos, seq, nvalid, obuf, S, H, G, D, Dv)
-#define GDT(DKV) do { if (in_bf16) GD(DKV, bf16); else GD(DKV, float); } while (0)
-    switch (DK) {
-        case 32: GDT(32); break;
-        case 64: GDT(64); break;
-        case 128: GDT(128); break;
-        default: GDT(256); break;
+    if (D > 256 || H % G != 0 || PS < (long)(2 * G + H) * D + H) return -1;
+    const long ntok = (long)B * S;
+    {
+        const long waves = ntok * (2 * G + H);
+        dim3 g0((unsigned)((waves + 3) / 4)), b0(4 * WAVE);
+        if (in_bf16) delta_prep_kernel<bf16><<<g0, b0, 0, st>>>(
+            qkv, cstride, (const bf16*)beta, bstride, (const bf16*)a, astride, dt_bias, a_log,
+            pos, seq, prep, PS, ntok, S, H, G, D);
+        else delta_prep_kernel<float><<<g0, b0, 0, st>>>(
+            qkv, cstride, (const float*)beta, bstride, (const float*)a, astride, dt_bias, a_log,
+            pos, seq, prep, PS, ntok, S, H, G, D);
+        int rc = (int)hipGetLastError();
+        if (rc) return rc;
     }
-#undef GDT
+    dim3 grid((Dv + GD_CW - 1) / GD_CW, H, B), block(GD_THREADS);
+#define GD(DKV, TCV) gated_delta_kernel<DKV, TCV><<<grid, block, 0, st>>>( \
+        qkv, cstride, prep, PS, state, pos, seq, nvalid, obuf, S, H, G, D, Dv)
+    if (D <= 32) GD(32, 16);
+    else if (D <= 64) GD(64, 16);
+    else if (D <= 128) GD(128, 16);
+    else GD(256, 8);
 #undef GD
     int rc = (int)hipGetLastError();
     if (rc) return rc;
-    const long waves = (long)B * S * H;
+    const long waves = ntok * H;
     dim3 g2((unsigned)((waves + 3) / 4)), b2(4 * WAVE);
     if (in_bf16) gated_rmsnorm_kernel<bf16><<<g2, b2, 0, st>>>(
-        obuf, (const bf16*)gate, gstride, norm_w, eps, pos, seq, (bf16*)out, (long)B * S, S, H, Dv);
+        obuf, (const bf16*)gate, gstride, norm_w, eps, pos, seq, (bf16*)out, ntok, S, H, Dv);
     else gated_rmsnorm_kernel<float><<<g2, b2, 0, st>>>(
-        obuf, (const float*)gate, gstride, norm_w, eps, pos, seq, (float*)out, (long)B * S, S, H, Dv);
+        obuf, (const float*)gate, gstride, norm_w, eps, pos, seq, (float*)out, ntok, S, H, Dv);
     return (int)hipGetLastError();
 }
 

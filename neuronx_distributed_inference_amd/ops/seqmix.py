@@ -234,12 +234,15 @@ def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps: float,
         assert beta.dtype == a.dtype == gate.dtype == out_dtype
         out = torch.empty(B, S, H * vdim, dtype=out_dtype, device=qkv.device)
         obuf = torch.empty(B, S, H * vdim, dtype=torch.float32, device=qkv.device)
+        PS = (2 * kv_heads + H) * dim + H
+        prep = torch.empty(B, S, PS, dtype=torch.float32, device=qkv.device)
         _check(lib.nx_gated_delta(
             _p(qkv), ctypes.c_long(_rows_view(qkv)), _p(beta),
             ctypes.c_long(_rows_view(beta)), _p(a), ctypes.c_long(_rows_view(a)),
             _p(gate), ctypes.c_long(_rows_view(gate)), _p(_f32(dt_bias)),
             _p(_f32(a_log)), _p(_f32(norm_w)), ctypes.c_float(eps), _p(state),
-            _p(step.positions), _p(step.seq_ids), _p(step.nvalid), _p(obuf), _p(out),
+            _p(step.positions), _p(step.seq_ids), _p(step.nvalid), _p(prep),
+            ctypes.c_long(PS), _p(obuf), _p(out),
             _is_bf16(beta), B, S, H, kv_heads, dim, vdim, _stream()),
             "gated_delta_rule")
         return out
