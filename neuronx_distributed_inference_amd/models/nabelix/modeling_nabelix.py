@@ -301,7 +301,7 @@ class NabelixForCausalLM(CausalLMBase):
             return sd[name].float()
 
         out["embed_tokens.weight"] = w("embed")
-        out["lm_head.weight"] = out["embed_tokens.weight"]
+        out["lm_head.weight"] = out["embed_tokens.weight"].clone()   # saved shards may not alias
         out["norm.weight"] = f("final.norm")
         for i, lc in enumerate(config.layers):
             s, d = f"l{i}.", f"layers.{i}."

@@ -537,3 +537,24 @@ def test_checkpoint_folder_and_schedule_replay(tmp_path):
     close(g0, wa[[0, 7]], 3e-4)
     close(g1, wb[[0]], 3e-4)
     close(g2, torch.stack([wb[8], wa[20]]), 3e-4)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_through_generate_adapter(device):
+    """The plain generate() entry point (no page table passed: the model
+    lays its slots out linearly over the page pool)."""
+    from neuronx_distributed_inference_amd.utils.hf_adapter import (
+        GenerationConfig,
+        HuggingFaceGenerationAdapter,
+    )
+
+    cfg = model_cfg()
+    W = make_weights(cfg, seed=15)
+    prompts = [tokens_for(cfg, 8, seed=40), tokens_for(cfg, 8, seed=41)]
+    want = [_oracle_greedy(cfg, W, p, 6) for p in prompts]
+    eng = make_engine(cfg, W, device, slots=2, page=4, pages=16, max_len=32)
+    model = eng.model
+    out = HuggingFaceGenerationAdapter(model).generate(
+        torch.tensor(prompts, device=device),
+        generation_config=GenerationConfig(max_new_tokens=6))
+    assert out[:, 8:].tolist() == want
