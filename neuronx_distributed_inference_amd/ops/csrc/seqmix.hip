@@ -416,6 +416,216 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
     }
 }
 
+// ------------------------------------- windowed biased attention, matrix cores
+// bf16 prompt-portion path. Workgroup = 64 query rows of one KV head (4 waves x
+// 16 rows: the group's heads x consecutive tokens); all waves walk the same
+// 64-key tiles, staged once in LDS (K row-major, V transposed). Scores are
+// computed transposed, S^T = K Q^T (mfma 16x16x32 bf16, fp32 accumulate), so a
+// lane ends up with 16 scores of ONE query row and the probabilities already
+// sit in the A-operand layout of the P.V product. Bias, mask and online softmax
+// are fp32 per lane; P enters the second product as a hi + lo bf16 pair (16
+// mantissa bits), V as stored.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+#define MA_ROWS 64
+#define MA_KT 64
+
+DEV uint16_t f2bf_rne(float f) {
+    uint32_t u = __float_as_uint(f);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+template <int DK, int DV>
+__global__ void __launch_bounds__(256)
+window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __restrict__ kc,
+                        const bf16* __restrict__ vc, const int* __restrict__ pos,
+                        const int* __restrict__ seq, const int* __restrict__ btab,
+                        int max_blocks, const float* __restrict__ r1,
+                        const float* __restrict__ r2, const bf16* __restrict__ gate,
+                        long gstride, bf16* __restrict__ out, int H, int G, int bsz, int S,
+                        float scale, int window, int keep, int QT) {
+    constexpr int KS = DK + 8;               // K tile row stride (elements)
+    constexpr int VS = MA_KT + 8;            // V^T tile row stride
+    __shared__ __attribute__((aligned(16))) uint16_t k_lds[MA_KT * KS];
+    __shared__ __attribute__((aligned(16))) uint16_t vt_lds[DV * VS];
+    __shared__ int rpos[MA_ROWS];
+    __shared__ float ra1[MA_ROWS], ra2[MA_ROWS];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
+    const int b = blockIdx.z, g = blockIdx.y, t0 = blockIdx.x * QT;
+    const int rep = H / G;
+    if (seq[b] < 0) return;
+    if (tid < MA_ROWS) {
+        const int tq = tid / rep, hh = tid % rep;
+        rpos[tid] = (tq < QT && t0 + tq < S) ? pos[(long)b * S + t0 + tq] : -1;
+        ra1[tid] = r1[g * rep + hh];
+        ra2[tid] = r2[g * rep + hh];
+    }
+    __syncthreads();
+    int i_min = 0x7fffffff, i_max = -1;
+    for (int r = 0; r < MA_ROWS; r += rep) {     // one entry per token
+        const int p = rpos[r];
+        if (p >= 0) { i_min = min(i_min, p); i_max = max(i_max, p); }
+    }
+    if (i_max < 0) return;                       // uniform
+    // this lane's query row (B operand of S^T): row = 16*wv + lr
+    const int myrow = wv * 16 + lr;
+    const int my_i = rpos[myrow];
+    const float a1 = ra1[myrow], a2 = ra2[myrow];
+    bf16x8_t qf[DK / 32];
+    {
+        const int tq = myrow / rep, h = g * rep + myrow % rep;
+        const bf16* qp = q + ((long)b * S + t0 + tq) * qstride + (long)h * DK;
+#pragma unroll
+        for (int ks = 0; ks < DK / 32; ++ks) {
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (my_i >= 0) raw = *reinterpret_cast<const uint4*>(qp + ks * 32 + lg * 8);
+            qf[ks] = *reinterpret_cast<bf16x8_t*>(&raw);
+        }
+    }
+    const int* bt = btab + (long)b * max_blocks;
+    const int lo = max(0, i_min - window + 1);
+    const int nfirst = min(keep, lo);
+    const int n = nfirst + (i_max - lo + 1);
+    const long krow = (long)G * DK, vrow = (long)G * DV;
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4_t o_acc[DV / 16];
+#pragma unroll
+    for (int nb = 0; nb < DV / 16; ++nb) o_acc[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int base = 0; base < n; base += MA_KT) {
+        // ---- stage K (row-major) and V (transposed) tiles
+        for (int c = tid; c < MA_KT * (DK / 8); c += 256) {
+            const int m = c / (DK / 8), part = c % (DK / 8);
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (base + m < n) {
+                const int mm = base + m;
+                const int j = mm < nfirst ? mm : lo + (mm - nfirst);
+                const int blk = bt[j / bsz];
+                const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
+                raw = *reinterpret_cast<const uint4*>(kc + slot * krow + (long)g * DK + part * 8);
+            }
+            *reinterpret_cast<uint4*>(k_lds + m * KS + part * 8) = raw;
+        }
+        for (int c = tid; c < MA_KT * (DV / 8); c += 256) {
+            const int m = c % MA_KT, part = c / MA_KT;   // consecutive lanes: consecutive keys
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (base + m < n) {
+                const int mm = base + m;
+                const int j = mm < nfirst ? mm : lo + (mm - nfirst);
+                const int blk = bt[j / bsz];
+                const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
+                raw = *reinterpret_cast<const uint4*>(vc + slot * vrow + (long)g * DV + part * 8);
+            }
+            const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                vt_lds[(part * 8 + 2 * e) * VS + m] = (uint16_t)(u[e] & 0xffffu);
+                vt_lds[(part * 8 + 2 * e + 1) * VS + m] = (uint16_t)(u[e] >> 16);
+            }
+        }
+        __syncthreads();
+        // ---- S^T = K Q^T: lane gets keys 16*kb + 4*lg + r of its own row lr
+        float sv[4][4];
+        float mt = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < DK / 32; ++ks) {
+                const bf16x8_t ka = *reinterpret_cast<const bf16x8_t*>(
+                    k_lds + (kb * 16 + lr) * KS + ks * 32 + lg * 8);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[ks], acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int mm = base + kb * 16 + lg * 4 + r;
+                const int j = mm < nfirst ? mm : lo + (mm - nfirst);
+                const int dist = my_i - j;
+                const bool vis = mm < n && my_i >= 0 && dist >= 0 && (dist < window || j < keep);
+                float x = -INFINITY;
+                if (vis) x = acc[r] * scale - a1 * __logf(1.f + a2 * (float)dist);
+                sv[kb][r] = x;
+                mt = fmaxf(mt, x);
+            }
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 16, WAVE));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, WAVE));
+        const float m_new = fmaxf(m_run, mt);
+        float corr = 1.f, psum = 0.f;
+        if (m_new > -INFINITY) {
+            corr = expf(m_run - m_new);
+#pragma unroll
+            for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float pv = sv[kb][r] > -INFINITY ? expf(sv[kb][r] - m_new) : 0.f;
+                    sv[kb][r] = pv;
+                    psum += pv;
+                }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sv[kb][r] = 0.f;
+        }
+        psum += __shfl_xor(psum, 16, WAVE);
+        psum += __shfl_xor(psum, 32, WAVE);
+        l_run = l_run * corr + psum;
+        m_run = m_new;
+        // ---- rescale O: its rows are 4*lg + r, their corr sits in lane (4*lg + r)
+        float cr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, lg * 4 + r, WAVE);
+#pragma unroll
+        for (int nb = 0; nb < DV / 16; ++nb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o_acc[nb][r] *= cr[r];
+        // ---- O += P V, 32 keys per product, P as hi + lo
+#pragma unroll
+        for (int kc2 = 0; kc2 < 2; ++kc2) {
+            union { bf16x8_t v; uint16_t u[8]; } ph, pl;
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) {
+                const float pv = sv[2 * kc2 + (jj >> 2)][jj & 3];
+                const uint16_t hb = f2bf_rne(pv);
+                ph.u[jj] = hb;
+                pl.u[jj] = f2bf_rne(pv - __uint_as_float((uint32_t)hb << 16));
+            }
+#pragma unroll
+            for (int nb = 0; nb < DV / 16; ++nb) {
+                union { bf16x8_t v; uint2 h[2]; } vb;
+                const uint16_t* vp = vt_lds + (nb * 16 + lr) * VS + 32 * kc2 + 4 * lg;
+                vb.h[0] = *reinterpret_cast<const uint2*>(vp);
+                vb.h[1] = *reinterpret_cast<const uint2*>(vp + 16);
+                o_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph.v, vb.v, o_acc[nb], 0, 0, 0);
+                o_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl.v, vb.v, o_acc[nb], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    // ---- epilogue: rows 4*lg + r of this wave, channel 16*nb + lr
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int row = wv * 16 + lg * 4 + r;
+        const float lsum = __shfl(l_run, lg * 4 + r, WAVE);
+        if (rpos[row] < 0) continue;
+        const int tq = row / rep, h = g * rep + row % rep;
+        const long tok = (long)b * S + t0 + tq;
+        const float inv = 1.f / lsum;
+        bf16* op = out + (tok * H + h) * (long)DV;
+        const bf16* gp = gate ? gate + tok * gstride + (long)h * DV : nullptr;
+#pragma unroll
+        for (int nb = 0; nb < DV / 16; ++nb) {
+            const int d = nb * 16 + lr;
+            float o = o_acc[nb][r] * inv;
+            if (gp) o *= sigmoidf_(__bfloat162float(gp[d]));
+            op[d] = __float2bfloat16(o);
+        }
+    }
+}
+
 // ------------------------------------------------------- gated delta rule
 // Three kernels per step.
 // (1) delta_prep_kernel, fully parallel over tokens: unit q and k per KV head
@@ -722,6 +932,26 @@ int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, 
     if ((long)B * S <= 0) return 0;
     if (Dv > WAVE * 4 || H % G != 0) return -1;
     if (!io_bf16 && out_bf16) return -2;
+    {
+        // matrix-core path: bf16 steps with prompt portions, common head shapes
+        const int rp = H / G;
+        const bool rep_ok = rp == 1 || rp == 2 || rp == 4 || rp == 8 || rp == 16;
+        const bool dk_ok = Dk == 64 || Dk == 128, dv_ok = Dv == 64 || Dv == 128;
+        if (io_bf16 && out_bf16 && S > 1 && rep_ok && dk_ok && dv_ok && (qstride % 8) == 0 &&
+            ((uintptr_t)q % 16) == 0) {
+            const int QTm = MA_ROWS / rp;
+            dim3 gm((S + QTm - 1) / QTm, G, B), bm(256);
+#define MA(DKV, DVV) window_attn_mfma_kernel<DKV, DVV><<<gm, bm, 0, st>>>( \
+        (const bf16*)q, qstride, (const bf16*)kc, (const bf16*)vc, pos, seq, btab, max_blocks, \
+        r1, r2, (const bf16*)gate, gstride, (bf16*)out, H, G, bsz, S, scale, window, keep, QTm)
+            if (Dk == 64 && Dv == 64) MA(64, 64);
+            else if (Dk == 64) MA(64, 128);
+            else if (Dv == 64) MA(128, 64);
+            else MA(128, 128);
+#undef MA
+            return (int)hipGetLastError();
+        }
+    }
     const bool dec = S == 1;                              // pure decode step
     const int NQ = dec ? 4 : 16, NW = dec ? 16 : 4;
     const int rep = H / G;

@@ -162,9 +162,10 @@ def tokens_for(cfg, n, seed):
     return torch.randint(0, cfg["vocab"], (n,), generator=g).tolist()
 
 
-def close(got, want, tol):
-    err = (got.double() - want.double()).abs().max().item()
-    assert err < tol, err
+def close(got, want, tol, rtol=0.0):
+    """|got - want| <= tol + rtol * |want| everywhere."""
+    excess = ((got.double() - want.double()).abs() - rtol * want.double().abs()).max().item()
+    assert excess < tol, excess
 
 
 # ----------------------------------------------------- mechanisms, alone
@@ -217,7 +218,7 @@ def test_short_conv_portions_and_slots(device, taps, act, residual):
         close(torch.cat(got[b]), want[b], 1e-5)
 
 
-def _attention_alone(device, L, T, spikes, page=4, cuts=None, dtype=F32, tol=2e-5):
+def _attention_alone(device, L, T, spikes, page=4, cuts=None, dtype=F32, tol=2e-5, rtol=0.0):
     """Attention core on its own paged cache. `spikes`: (query i, key j) pairs
     whose score is made to dominate if (and only if) the mask lets it."""
     torch.manual_seed(3)
@@ -237,6 +238,8 @@ def _attention_alone(device, L, T, spikes, page=4, cuts=None, dtype=F32, tol=2e-
         q[i] += 6.0 * d
     v = h @ W["v"].T
     gate = h @ W["g"].T
+    if dtype != F32:      # both sides see the values the kernel is given
+        q, k, v, gate = (t.to(dtype).double() for t in (q, k, v, gate))
     # oracle with the same (spiked) q/k: feed them through identity projections
     hq = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v, gate], 1)
     o0, o1, o2 = H * D, H * D + G * D, H * D + G * D + G * Dv
@@ -266,7 +269,7 @@ def _attention_alone(device, L, T, spikes, page=4, cuts=None, dtype=F32, tol=2e-
                 gate=gate[sl].view(1, n, -1).to(device, dtype))
         got.append(y[0].float().cpu())
         at += n
-    close(torch.cat(got), want, tol)
+    close(torch.cat(got), want, tol, rtol)
 
 
 EDGE = left_cfg(heads=4, kv_heads=2, dim=8, vdim=16, size=7, keep=3, scale=0.5)
@@ -298,7 +301,22 @@ def test_attention_other_shapes(device, L):
 def test_attention_bf16_long_window_gpu():
     L = left_cfg(8, 2, 64, 128, size=200, keep=20, scale=0.1)
     _attention_alone("cuda", L, 300, [(290, 91), (290, 90), (299, 19)], page=64,
-                     cuts=[150, 1, 1, 148], dtype=torch.bfloat16, tol=0.08)
+                     cuts=[150, 1, 1, 148], dtype=torch.bfloat16, tol=0.01, rtol=0.01)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("L,cuts", [
+    (left_cfg(4, 2, 64, 64, size=7, keep=3, scale=0.5), None),
+    (left_cfg(4, 2, 64, 64, size=7, keep=3, scale=0.5), [5, 9, 2, 17]),
+    (left_cfg(8, 1, 128, 64, size=40, keep=0, scale=0.3), [3, 30]),
+    (left_cfg(2, 2, 64, 128, size=100, keep=6, scale=0.3), [33]),
+    (left_cfg(16, 1, 128, 128, size=20, keep=2, scale=0.2), [20, 13]),
+])
+def test_attention_edges_bf16_matrix_path_gpu(L, cuts):
+    """bf16 prompt portions with common head shapes take the matrix-core
+    kernel: same spiked edges (window, kept-first, page border, far)."""
+    _attention_alone("cuda", L, 33, EDGE_SPIKES, page=8, cuts=cuts,
+                     dtype=torch.bfloat16, tol=0.01, rtol=0.01)
 
 
 def _delta_alone(device, R, T, cuts, slots=(1,), eps=1e-4):
