@@ -935,8 +935,9 @@ int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, 
     {
         // matrix-core path: bf16 steps with prompt portions, common head shapes
         const int rp = H / G;
-        const bool rep_ok = rp == 1 || rp == 2 || rp == 4 || rp == 8 || rp == 16;
-        const bool dk_ok = Dk == 64 || Dk == 128, dv_ok = Dv == 64 || Dv == 128;
+        const bool rep_ok = rp <= MA_ROWS;       // rows beyond QT*rep stay idle
+        const bool dk_ok = Dk == 32 || Dk == 64 || Dk == 128;
+        const bool dv_ok = Dv == 32 || Dv == 64 || Dv == 128;
         if (io_bf16 && out_bf16 && S > 1 && rep_ok && dk_ok && dv_ok && (qstride % 8) == 0 &&
             ((uintptr_t)q % 16) == 0) {
             const int QTm = MA_ROWS / rp;
@@ -944,10 +945,11 @@ int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, 
 #define MA(DKV, DVV) window_attn_mfma_kernel<DKV, DVV><<<gm, bm, 0, st>>>( \
         (const bf16*)q, qstride, (const bf16*)kc, (const bf16*)vc, pos, seq, btab, max_blocks, \
         r1, r2, (const bf16*)gate, gstride, (bf16*)out, H, G, bsz, S, scale, window, keep, QTm)
-            if (Dk == 64 && Dv == 64) MA(64, 64);
-            else if (Dk == 64) MA(64, 128);
-            else if (Dv == 64) MA(128, 64);
-            else MA(128, 128);
+#define MAV(DKV) do { if (Dv == 32) MA(DKV, 32); else if (Dv == 64) MA(DKV, 64); else MA(DKV, 128); } while (0)
+            if (Dk == 32) MAV(32);
+            else if (Dk == 64) MAV(64);
+            else MAV(128);
+#undef MAV
 #undef MA
             return (int)hipGetLastError();
         }

@@ -311,6 +311,8 @@ def test_attention_bf16_long_window_gpu():
     (left_cfg(8, 1, 128, 64, size=40, keep=0, scale=0.3), [3, 30]),
     (left_cfg(2, 2, 64, 128, size=100, keep=6, scale=0.3), [33]),
     (left_cfg(16, 1, 128, 128, size=20, keep=2, scale=0.2), [20, 13]),
+    (left_cfg(6, 2, 32, 128, size=9, keep=4, scale=0.4), [2, 31]),
+    (left_cfg(5, 1, 64, 32, size=12, keep=1, scale=0.4), [16, 16, 1]),
 ])
 def test_attention_edges_bf16_matrix_path_gpu(L, cuts):
     """bf16 prompt portions with common head shapes take the matrix-core
