@@ -670,6 +670,16 @@ __global__ void delta_prep_kernel(const float* __restrict__ qkv, long cstride,
         float inv = 1.f / sqrtf(wave_sum(ss) + 1e-6f);
         if (u < G) inv *= 1.f / sqrtf((float)D);
         for (int i = lane; i < D; i += WAVE) pr[(long)u * D + i] = src[i] * inv;
+        if (u < G) {
+            // q^ . k^ of this KV head: lets the scan read out before it writes
+            const float* ksrc = src + (long)G * D;
+            float sk = 0.f, qk = 0.f;
+            for (int i = lane; i < D; i += WAVE) { float y = ksrc[i]; sk += y * y; qk += src[i] * y; }
+            sk = wave_sum(sk);
+            qk = wave_sum(qk);
+            if (lane == 0)
+                pr[(long)(2 * G + H) * D + H + u] = qk * inv * (1.f / sqrtf(sk + 1e-6f));
+        }
     } else {
         const int h = u - 2 * G;
         const float neg_rate = -expf(a_log[h]);
@@ -682,6 +692,20 @@ __global__ void delta_prep_kernel(const float* __restrict__ qkv, long cstride,
     }
 }
 
+// sum over the 8 adjacent lanes that share a value channel, on the DPP path
+// (quad xor 1, quad xor 2, then the mirrored half row: after the first two
+// steps every lane of a quad holds the quad's sum, so any lane of the other
+// quad will do)
+DEV float part_sum8(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+        0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+        0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+        0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+    return v;
+}
+
 template <int DK, int TC>
 __global__ void __launch_bounds__(GD_THREADS)
 gated_delta_kernel(const float* __restrict__ qkv, long cstride, const float* __restrict__ prep,
@@ -691,7 +715,7 @@ gated_delta_kernel(const float* __restrict__ qkv, long cstride, const float* __r
     constexpr int R = DK / GD_PARTS;         // rows per lane
     constexpr int F = R / 4;                 // float4s per lane
     constexpr int NQKG = 3 * TC * DK;        // LDS floats per chunk: q | k | decay
-    constexpr int NE = NQKG + TC * GD_CW + TC;   // ... | v (TC x GD_CW) | beta (TC)
+    constexpr int NE = NQKG + TC * GD_CW + 2 * TC;   // ... | v (TC x GD_CW) | beta | q.k
     constexpr int PER = (NE + GD_THREADS - 1) / GD_THREADS;
     __shared__ __attribute__((aligned(16))) float buf[PER * GD_THREADS];
     const float* qs = buf;
@@ -699,6 +723,7 @@ gated_delta_kernel(const float* __restrict__ qkv, long cstride, const float* __r
     const float* gs = buf + 2 * TC * DK;
     const float* vs = buf + NQKG;
     const float* bs = vs + TC * GD_CW;
+    const float* kqs = bs + TC;
     const int h = blockIdx.y, b = blockIdx.z;
     const int slot = seq[b];
     const int n = nvalid[b];
@@ -722,6 +747,7 @@ gated_delta_kernel(const float* __restrict__ qkv, long cstride, const float* __r
         }
     const long off_q = (long)g * D, off_k = (long)(G + g) * D, off_g = (long)(2 * G + h) * D;
     const long off_b = (long)(2 * G + H) * D + h;
+    const long off_kq = (long)(2 * G + H) * D + H + g;
     const long off_v = 2L * G * D + (long)h * Dv + col0;
 
     float pre[PER];
@@ -742,8 +768,9 @@ gated_delta_kernel(const float* __restrict__ qkv, long cstride, const float* __r
                 const int tk = (idx - NQKG) / GD_CW, c = (idx - NQKG) % GD_CW;            \
                 if (tk < ftc && col0 + c < Dv) v = qkv[(frow + tk) * cstride + off_v + c]; \
             } else if (idx < NE) {                                                        \
-                const int tk = idx - NQKG - TC * GD_CW;                                   \
-                if (tk < ftc) v = prep[(frow + tk) * PS + off_b];                         \
+                const int e = idx - NQKG - TC * GD_CW;                                    \
+                const int tk = e % TC;                                                    \
+                if (tk < ftc) v = prep[(frow + tk) * PS + (e < TC ? off_b : off_kq)];     \
             }                                                                             \
             pre[x] = v;                                                                   \
         }                                                                                 \
@@ -761,31 +788,30 @@ gated_delta_kernel(const float* __restrict__ qkv, long cstride, const float* __r
             const float4* k4 = reinterpret_cast<const float4*>(ks + tk * DK) + part;
             const float4* q4 = reinterpret_cast<const float4*>(qs + tk * DK) + part;
             float4 kk[F];
-            float dot = 0.f;
+            float dot = 0.f, oq = 0.f;       // (dS)^T k and (dS)^T q, this lane's rows
 #pragma unroll
             for (int f = 0; f < F; ++f) {
                 const float4 gg = g4[f * GD_PARTS];
+                const float4 qq = q4[f * GD_PARTS];
                 kk[f] = k4[f * GD_PARTS];
-                s[4 * f] *= gg.x; dot += s[4 * f] * kk[f].x;
-                s[4 * f + 1] *= gg.y; dot += s[4 * f + 1] * kk[f].y;
-                s[4 * f + 2] *= gg.z; dot += s[4 * f + 2] * kk[f].z;
-                s[4 * f + 3] *= gg.w; dot += s[4 * f + 3] * kk[f].w;
+                s[4 * f] *= gg.x; dot += s[4 * f] * kk[f].x; oq += s[4 * f] * qq.x;
+                s[4 * f + 1] *= gg.y; dot += s[4 * f + 1] * kk[f].y; oq += s[4 * f + 1] * qq.y;
+                s[4 * f + 2] *= gg.z; dot += s[4 * f + 2] * kk[f].z; oq += s[4 * f + 2] * qq.z;
+                s[4 * f + 3] *= gg.w; dot += s[4 * f + 3] * kk[f].w; oq += s[4 * f + 3] * qq.w;
             }
-#pragma unroll
-            for (int o = GD_PARTS / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o, WAVE);
+            dot = part_sum8(dot);
+            oq = part_sum8(oq);
             const float u = bs[tk] * (vs[tk * GD_CW + cl] - dot);
-            float o = 0.f;
+            // read-out of the updated state: (dS + k u^T)^T q = (dS)^T q + u (k.q)
+            if (act && part == 0)
+                obuf[((row0 + tk) * H + h) * (long)Dv + col] = oq + u * kqs[tk];
 #pragma unroll
             for (int f = 0; f < F; ++f) {
-                const float4 qq = q4[f * GD_PARTS];
-                s[4 * f] += kk[f].x * u; o += s[4 * f] * qq.x;
-                s[4 * f + 1] += kk[f].y * u; o += s[4 * f + 1] * qq.y;
-                s[4 * f + 2] += kk[f].z * u; o += s[4 * f + 2] * qq.z;
-                s[4 * f + 3] += kk[f].w * u; o += s[4 * f + 3] * qq.w;
+                s[4 * f] += kk[f].x * u;
+                s[4 * f + 1] += kk[f].y * u;
+                s[4 * f + 2] += kk[f].z * u;
+                s[4 * f + 3] += kk[f].w * u;
             }
-#pragma unroll
-            for (int x = GD_PARTS / 2; x > 0; x >>= 1) o += __shfl_xor(o, x, WAVE);
-            if (act && part == 0) obuf[((row0 + tk) * H + h) * (long)Dv + col] = o;
         }
         __syncthreads();
     }
@@ -987,7 +1013,7 @@ int nx_gated_delta(const float* qkv, long cstride, const void* beta, long bstrid
                    float* obuf, void* out, int in_bf16, int B, int S, int H, int G, int D,
                    int Dv, hipStream_t st) {
     if (B <= 0 || S <= 0) return 0;
-    if (D > 256 || H % G != 0 || PS < (long)(2 * G + H) * D + H) return -1;
+    if (D > 256 || H % G != 0 || PS < (long)(2 * G + H) * D + H + G) return -1;
     const long ntok = (long)B * S;
     {
         const long waves = ntok * (2 * G + H);

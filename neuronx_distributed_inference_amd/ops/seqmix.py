@@ -234,7 +234,7 @@ def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps: float,
         assert beta.dtype == a.dtype == gate.dtype == out_dtype
         out = torch.empty(B, S, H * vdim, dtype=out_dtype, device=qkv.device)
         obuf = torch.empty(B, S, H * vdim, dtype=torch.float32, device=qkv.device)
-        PS = (2 * kv_heads + H) * dim + H
+        PS = (2 * kv_heads + H) * dim + H + kv_heads
         prep = torch.empty(B, S, PS, dtype=torch.float32, device=qkv.device)
         _check(lib.nx_gated_delta(
             _p(qkv), ctypes.c_long(_rows_view(qkv)), _p(beta),
