@@ -633,10 +633,10 @@ window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __
 //     per head and key channel, beta = sigmoid(.), all fp32, into one row per
 //     token: [q (G*D) | k (G*D) | decay (H*D) | beta (H)], stride PS.
 // (2) gated_delta_kernel, the serial scan. Workgroup = (row, head, block of
-//     GD_CW value channels), 256 threads. The (D x Dv) state is kept in
-//     registers: GD_PARTS adjacent lanes share one value channel (column) and
-//     split its D rows in float4-interleaved order, so a token costs
-//     D/GD_PARTS multiply-adds per lane plus two 3-step lane reductions and no
+//     value channels), 256 threads. The (D x Dv) state is kept in registers:
+//     16 (8 for D <= 32) adjacent lanes share one value channel (column) and
+//     split its D rows in float4-interleaved order, so a token costs D/16
+//     multiply-adds per lane plus two DPP lane reductions and no
 //     workgroup-wide traffic. Tokens go in chunks of TC through LDS; the next
 //     chunk's rows are fetched into registers while the current one is
 //     scanned. State memory layout is (slot, head, Dv, D): a lane's rows are
@@ -644,8 +644,6 @@ window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __
 // (3) gated_rmsnorm_kernel: per-head RMS norm, weight and sigmoid gate (needs
 //     all value channels of a head, which (2) spreads over workgroups).
 #define GD_THREADS 256
-#define GD_PARTS 8
-#define GD_CW (GD_THREADS / GD_PARTS)
 
 template <typename T>
 __global__ void delta_prep_kernel(const float* __restrict__ qkv, long cstride,
@@ -692,26 +690,31 @@ __global__ void delta_prep_kernel(const float* __restrict__ qkv, long cstride,
     }
 }
 
-// sum over the 8 adjacent lanes that share a value channel, on the DPP path
-// (quad xor 1, quad xor 2, then the mirrored half row: after the first two
-// steps every lane of a quad holds the quad's sum, so any lane of the other
-// quad will do)
-DEV float part_sum8(float v) {
+// sum over the 8 or 16 adjacent lanes that share a value channel, on the DPP
+// path (quad xor 1, quad xor 2, mirrored half row, mirrored row: after each
+// step every lane of a group holds the group's sum, so any lane of the
+// sibling group will do)
+template <int PARTS>
+DEV float part_sum(float v) {
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
         0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
         0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
         0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+    if (PARTS == 16)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+            0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));   // row_mirror
     return v;
 }
 
-template <int DK, int TC>
+template <int DK, int TC, int GD_PARTS>
 __global__ void __launch_bounds__(GD_THREADS)
 gated_delta_kernel(const float* __restrict__ qkv, long cstride, const float* __restrict__ prep,
                    long PS, float* __restrict__ state, const int* __restrict__ pos,
                    const int* __restrict__ seq, const int* __restrict__ nvalid,
                    float* __restrict__ obuf, int S, int H, int G, int D, int Dv) {
+    constexpr int GD_CW = GD_THREADS / GD_PARTS;   // value channels per workgroup
     constexpr int R = DK / GD_PARTS;         // rows per lane
     constexpr int F = R / 4;                 // float4s per lane
     constexpr int NQKG = 3 * TC * DK;        // LDS floats per chunk: q | k | decay
@@ -783,6 +786,7 @@ gated_delta_kernel(const float* __restrict__ qkv, long cstride, const float* __r
         for (int x = 0; x < PER; ++x) buf[tid + x * GD_THREADS] = pre[x];
         __syncthreads();
         if (t0 + TC < n) GD_FETCH(t0 + TC)   // in flight during the scan below
+#pragma unroll 2
         for (int tk = 0; tk < tc; ++tk) {
             const float4* g4 = reinterpret_cast<const float4*>(gs + tk * DK) + part;
             const float4* k4 = reinterpret_cast<const float4*>(ks + tk * DK) + part;
@@ -799,8 +803,8 @@ gated_delta_kernel(const float* __restrict__ qkv, long cstride, const float* __r
                 s[4 * f + 2] *= gg.z; dot += s[4 * f + 2] * kk[f].z; oq += s[4 * f + 2] * qq.z;
                 s[4 * f + 3] *= gg.w; dot += s[4 * f + 3] * kk[f].w; oq += s[4 * f + 3] * qq.w;
             }
-            dot = part_sum8(dot);
-            oq = part_sum8(oq);
+            dot = part_sum<GD_PARTS>(dot);
+            oq = part_sum<GD_PARTS>(oq);
             const float u = bs[tk] * (vs[tk * GD_CW + cl] - dot);
             // read-out of the updated state: (dS + k u^T)^T q = (dS)^T q + u (k.q)
             if (act && part == 0)
@@ -1027,13 +1031,15 @@ int nx_gated_delta(const float* qkv, long cstride, const void* beta, long bstrid
         int rc = (int)hipGetLastError();
         if (rc) return rc;
     }
-    dim3 grid((Dv + GD_CW - 1) / GD_CW, H, B), block(GD_THREADS);
-#define GD(DKV, TCV) gated_delta_kernel<DKV, TCV><<<grid, block, 0, st>>>( \
+    const int parts = D <= 32 ? 8 : 16;
+    const int cw = GD_THREADS / parts;
+    dim3 grid((Dv + cw - 1) / cw, H, B), block(GD_THREADS);
+#define GD(DKV, TCV, PV) gated_delta_kernel<DKV, TCV, PV><<<grid, block, 0, st>>>( \
         qkv, cstride, prep, PS, state, pos, seq, nvalid, obuf, S, H, G, D, Dv)
-    if (D <= 32) GD(32, 16);
-    else if (D <= 64) GD(64, 16);
-    else if (D <= 128) GD(128, 16);
-    else GD(256, 8);
+    if (D <= 32) GD(32, 16, 8);
+    else if (D <= 64) GD(64, 16, 16);
+    else if (D <= 128) GD(128, 16, 16);
+    else GD(256, 8, 16);
 #undef GD
     int rc = (int)hipGetLastError();
     if (rc) return rc;
