@@ -87,17 +87,17 @@ __global__ void short_conv_kernel(const TIn* __restrict__ x, const float* __rest
                                   const float* __restrict__ tail, const int* __restrict__ pos,
                                   const int* __restrict__ seq, TOut* __restrict__ y,
                                   int B, int S, int C, int taps, int act_silu, int residual) {
-    const long total = (long)B * S * C;
+    // one token per blockIdx.x (no divisions on the hot path), channels along y
     const int R = taps - 1;
-    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (long)gridDim.x * blockDim.x) {
-        const int c = idx % C;
-        const long bt = idx / C;
-        const int t = bt % S;
-        const int b = bt / S;
-        const int p = pos[bt];
-        const int slot = seq[b];
-        if (p < 0 || slot < 0) { stf<TOut>(y + idx, 0.f); continue; }
+    const long bt = blockIdx.x;
+    const int t = (int)(bt % S);
+    const int b = (int)(bt / S);
+    const int p = pos[bt];
+    const int slot = seq[b];
+    const bool live = p >= 0 && slot >= 0;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
+        const long idx = bt * C + c;
+        if (!live) { stf<TOut>(y + idx, 0.f); continue; }
         const float* wr = w + (long)c * taps;
         float acc = 0.f;
         for (int j = 0; j < taps; ++j) {
@@ -916,7 +916,9 @@ int nx_short_conv(const void* x, int x_bf16, const float* w, const float* tail, 
                   int act_silu, int residual, hipStream_t st) {
     const long total = (long)B * S * C;
     if (total <= 0) return 0;
-    dim3 grid(grid_for(total, 256)), block(256);
+    if ((long)B * S > 2147483647L) return -1;
+    const int cy = (C + 255) / 256;
+    dim3 grid((unsigned)((long)B * S), cy > 65535 ? 65535 : cy), block(256);
 #define SC(TI, TO) short_conv_kernel<TI, TO><<<grid, block, 0, st>>>( \
         (const TI*)x, w, tail, pos, seq, (TO*)y, B, S, C, taps, act_silu, residual)
     if (x_bf16 && y_bf16) SC(bf16, bf16);
