@@ -145,11 +145,10 @@ def short_conv(x, w, tail, step: StepLayout, activation: str = "none",
     ref.short_conv). Does not advance the tail: call short_conv_commit."""
     if x.is_cuda:
         lib = _load()
-        x = x.contiguous()
         B, S, C = x.shape
         y = torch.empty(B, S, C, dtype=out_dtype, device=x.device)
         _check(lib.nx_short_conv(
-            _p(x), _is_bf16(x), _p(_f32(w)), _p(tail), _p(step.positions),
+            _p(x), ctypes.c_long(_rows_view(x)), _is_bf16(x), _p(_f32(w)), _p(tail), _p(step.positions),
             _p(step.seq_ids), _p(y), _is_bf16(y), B, S, C, w.shape[1],
             int(activation == "silu"), int(residual), _stream()), "short_conv")
         return y
@@ -160,11 +159,10 @@ def short_conv(x, w, tail, step: StepLayout, activation: str = "none",
 def short_conv_commit(x, tail, step: StepLayout):
     if x.is_cuda:
         lib = _load()
-        x = x.contiguous()
         B, S, C = x.shape
         assert tail.dtype == torch.float32 and tail.is_contiguous()
         _check(lib.nx_short_conv_commit(
-            _p(x), _is_bf16(x), _p(tail), _p(step.positions), _p(step.seq_ids),
+            _p(x), ctypes.c_long(_rows_view(x)), _is_bf16(x), _p(tail), _p(step.positions), _p(step.seq_ids),
             _p(step.nvalid), B, S, C, tail.shape[1], _stream()), "short_conv_commit")
         return
     ref.short_conv_commit(x, tail, step.positions, step.seq_ids)
