@@ -82,75 +82,44 @@ layer_norm_kernel(const float* __restrict__ x, const float* __restrict__ w,
 // ------------------------------------------------------------- short conv
 // y[b,t,c] = act(sum_j w[c,j] * x[b, t-R+j, c]) (+ x[b,t,c]); columns before
 // the step come from the carried tail (oldest first), positions < 0 are zero
-// 8 consecutive channels of one token as floats (row-strided input allowed)
-template <typename T> DEV void ld8(const T* p, float* v);
-template <> DEV void ld8<bf16>(const bf16* p, float* v) {
-    const uint4 raw = *reinterpret_cast<const uint4*>(p);
-    const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        v[2 * e] = __uint_as_float(u[e] << 16);
-        v[2 * e + 1] = __uint_as_float(u[e] & 0xffff0000u);
-    }
-}
-template <> DEV void ld8<float>(const float* p, float* v) {
-    const float4 a = *reinterpret_cast<const float4*>(p);
-    const float4 b = *reinterpret_cast<const float4*>(p + 4);
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-}
-
-// one token per blockIdx.x (no divisions on the hot path), channels along y;
-// VEC = 8 channels per thread when the layout allows 16-byte accesses, else 1.
+// y[b,t,c] = act(sum_j w[c,j] * x[b, t-R+j, c]) (+ x[b,t,c]); columns before
+// the step come from the carried tail (oldest first), positions < 0 are zero.
 // `xs` is the input's row stride in elements (a column slice of a wider
-// projection is read in place); y is dense.
-template <typename TIn, typename TOut, int VEC>
+// projection is read in place); y is dense. One thread per element: adjacent
+// lanes read adjacent channels of the same row for every tap.
+template <typename TIn, typename TOut>
 __global__ void short_conv_kernel(const TIn* __restrict__ x, long xs, const float* __restrict__ w,
                                   const float* __restrict__ tail, const int* __restrict__ pos,
                                   const int* __restrict__ seq, TOut* __restrict__ y,
                                   int B, int S, int C, int taps, int act_silu, int residual) {
+    const long total = (long)B * S * C;
     const int R = taps - 1;
-    const long bt = blockIdx.x;
-    const int t = (int)(bt % S);
-    const int b = (int)(bt / S);
-    const int p = pos[bt];
-    const int slot = seq[b];
-    const bool live = p >= 0 && slot >= 0;
-    for (int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC; c < C;
-         c += gridDim.y * blockDim.x * VEC) {
-        float acc[VEC];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
-        if (live) {
-            float cur[VEC];
-            for (int j = 0; j < taps; ++j) {
-                const int col = t - R + j;
-                float xv[VEC];
-                if (col >= 0) {
-                    const TIn* xp = x + ((long)b * S + col) * xs + c;
-                    if constexpr (VEC == 8) ld8<TIn>(xp, xv); else xv[0] = ldf<TIn>(xp);
-                } else {
-                    const int ps = p - R + j;              // source position
-                    const float* tp = tail + ((long)slot * R + (R + col)) * C + c;
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) xv[e] = ps < 0 ? 0.f : tp[e];
-                }
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) acc[e] += w[(long)(c + e) * taps + j] * xv[e];
-                if (j == taps - 1) {
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) cur[e] = xv[e];
-                }
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int c = idx % C;
+        const long bt = idx / C;
+        const int t = bt % S;
+        const int b = bt / S;
+        const int p = pos[bt];
+        const int slot = seq[b];
+        if (p < 0 || slot < 0) { stf<TOut>(y + idx, 0.f); continue; }
+        const float* wr = w + (long)c * taps;
+        float acc = 0.f, cur = 0.f;
+        for (int j = 0; j < taps; ++j) {
+            const int col = t - R + j;
+            float xv;
+            if (col >= 0) {
+                xv = ldf<TIn>(x + ((long)b * S + col) * xs + c);
+            } else {
+                const int ps = p - R + j;              // source position
+                xv = ps < 0 ? 0.f : tail[((long)slot * R + (R + col)) * C + c];
             }
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                if (act_silu) acc[e] = acc[e] * sigmoidf_(acc[e]);
-                if (residual) acc[e] += cur[e];
-            }
+            acc += wr[j] * xv;
+            cur = xv;
         }
-        TOut* yp = y + bt * C + c;
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) stf<TOut>(yp + e, acc[e]);
+        if (act_silu) acc = acc * sigmoidf_(acc);
+        if (residual) acc += cur;
+        stf<TOut>(y + idx, acc);
     }
 }
 
@@ -954,19 +923,9 @@ int nx_short_conv(const void* x, long xs, int x_bf16, const float* w, const floa
                   int taps, int act_silu, int residual, hipStream_t st) {
     const long total = (long)B * S * C;
     if (total <= 0) return 0;
-    if ((long)B * S > 2147483647L) return -1;
-    // 16-byte input accesses need 8-channel groups that stay aligned on every row
-    const int esz = x_bf16 ? 2 : 4;
-    const bool vec = (C % 8) == 0 && ((xs * esz) % 16) == 0 && ((uintptr_t)x % 16) == 0;
-    const int per = vec ? 8 : 1;
-    const int cy = (C / per + 255) / 256;
-    dim3 grid((unsigned)((long)B * S), cy > 65535 ? 65535 : (cy < 1 ? 1 : cy)), block(256);
-#define SC(TI, TO) do { \
-        if (vec) short_conv_kernel<TI, TO, 8><<<grid, block, 0, st>>>( \
-            (const TI*)x, xs, w, tail, pos, seq, (TO*)y, B, S, C, taps, act_silu, residual); \
-        else short_conv_kernel<TI, TO, 1><<<grid, block, 0, st>>>( \
-            (const TI*)x, xs, w, tail, pos, seq, (TO*)y, B, S, C, taps, act_silu, residual); \
-    } while (0)
+    dim3 grid(grid_for(total, 256)), block(256);
+#define SC(TI, TO) short_conv_kernel<TI, TO><<<grid, block, 0, st>>>( \
+        (const TI*)x, xs, w, tail, pos, seq, (TO*)y, B, S, C, taps, act_silu, residual)
     if (x_bf16 && y_bf16) SC(bf16, bf16);
     else if (x_bf16) SC(bf16, float);
     else if (y_bf16) SC(float, bf16);
