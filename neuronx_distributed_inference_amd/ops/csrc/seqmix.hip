@@ -900,6 +900,34 @@ __global__ void gelu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, l
     }
 }
 
+// 8 channels per thread, 16-byte accesses; rows on blockIdx.y (strided)
+template <typename T>
+__global__ void gelu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, long rows,
+                                    int I) {
+    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (c >= I) return;
+    for (long r = blockIdx.y; r < rows; r += gridDim.y) {
+        float z[8], u[8], o[8];
+        load8<T>(gu + r * 2 * I + c, z);
+        load8<T>(gu + r * 2 * I + I + c, u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            o[e] = 0.5f * z[e] * (1.f + tanhf(0.7978845608028654f *
+                                              (z[e] + 0.044715f * z[e] * z[e] * z[e]))) * u[e];
+        T* op = out + r * I + c;
+        if constexpr (sizeof(T) == 2) {
+            uint32_t pk[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                pk[e] = (uint32_t)f2bf_rne(o[2 * e]) | ((uint32_t)f2bf_rne(o[2 * e + 1]) << 16);
+            *reinterpret_cast<uint4*>(op) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        } else {
+            *reinterpret_cast<float4*>(op) = make_float4(o[0], o[1], o[2], o[3]);
+            *reinterpret_cast<float4*>(op + 4) = make_float4(o[4], o[5], o[6], o[7]);
+        }
+    }
+}
+
 // =================================================================== C ABI
 static inline int grid_for(long total, int block, int cap = 8192) {
     long g = (total + block - 1) / block;
@@ -1081,6 +1109,12 @@ int nx_residual_add(float* x, const void* a, float sa, const void* b, float sb, 
 
 int nx_gelu_mul(const void* gu, void* out, int is_bf16, long rows, int I, hipStream_t st) {
     if (rows <= 0) return 0;
+    if ((I % 8) == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+        dim3 gv((I / 8 + 255) / 256, (unsigned)(rows > 32768 ? 32768 : rows)), bv(256);
+        if (is_bf16) gelu_mul_vec_kernel<bf16><<<gv, bv, 0, st>>>((const bf16*)gu, (bf16*)out, rows, I);
+        else gelu_mul_vec_kernel<float><<<gv, bv, 0, st>>>((const float*)gu, (float*)out, rows, I);
+        return (int)hipGetLastError();
+    }
     dim3 grid(grid_for(rows * I, 256)), block(256);
     if (is_bf16) gelu_mul_kernel<bf16><<<grid, block, 0, st>>>((const bf16*)gu, (bf16*)out, rows, I);
     else gelu_mul_kernel<float><<<grid, block, 0, st>>>((const float*)gu, (float*)out, rows, I);

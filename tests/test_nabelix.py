@@ -179,6 +179,20 @@ def test_layer_norm_op(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("ff", [12, 16, 40])          # scalar and 8-wide kernel paths
+def test_gelu_mul_and_residual_ops(device, ff):
+    torch.manual_seed(16)
+    gu = torch.randn(5, 2 * ff) * 2
+    want = oracle.gelu_tanh(gu[:, :ff].double()) * gu[:, ff:].double()
+    close(seqmix.gelu_tanh_mul_fused(gu.to(device)).cpu(), want, 1e-5)
+    x, a, b = torch.randn(3, 7), torch.randn(3, 7), torch.randn(3, 7)
+    got = seqmix.residual_add(x.clone().to(device), a.to(device), 1.25, b.to(device), 0.5).cpu()
+    close(got, x.double() + 1.25 * a.double() + 0.5 * b.double(), 1e-5)
+    lg = torch.randn(4, 9) * 40
+    close(seqmix.softcap(lg.to(device), 30.0).cpu(), 30.0 * torch.tanh(lg.double() / 30.0), 1e-4)
+
+
+@pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("taps", [1, 2, 4])
 @pytest.mark.parametrize("act,residual", [("none", True), ("silu", False)])
 def test_short_conv_portions_and_slots(device, taps, act, residual):
