@@ -44,6 +44,25 @@ DEV float wave_max(float v) {
 DEV float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
 DEV float softplusf_(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
+// 8 consecutive elements as floats, one or two 16-byte loads
+template <typename T> DEV void load8(const T* p, float* v);
+template <> DEV void load8<bf16>(const bf16* p, float* v) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(p);
+    const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        v[2 * e] = __uint_as_float(u[e] << 16);
+        v[2 * e + 1] = __uint_as_float(u[e] & 0xffff0000u);
+    }
+}
+template <> DEV void load8<float>(const float* p, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    const float4 b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+
 // ---------------------------------------------------------------- LayerNorm
 // one 256-thread workgroup per row; mean, then variance of the deviations
 // (both fp32); the row is re-read from cache, not kept in registers, so any
@@ -123,6 +142,95 @@ __global__ void short_conv_kernel(const TIn* __restrict__ x, long xs, const floa
     }
 }
 
+// Tiled variant for the common filter lengths: a thread owns 8 adjacent
+// channels, keeps their taps in registers and walks SC_TT consecutive tokens
+// with a sliding window of the last TAPS-1 inputs, so every input element is
+// loaded once (16 bytes per load) instead of TAPS times.
+#define SC_TT 16
+
+template <typename T> DEV void st8(T* p, const float* v);
+template <> DEV void st8<float>(float* p, const float* v) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+
+template <typename TIn, typename TOut, int TAPS>
+__global__ void short_conv_tile_kernel(const TIn* __restrict__ x, long xs,
+                                       const float* __restrict__ w,
+                                       const float* __restrict__ tail,
+                                       const int* __restrict__ pos, const int* __restrict__ seq,
+                                       const int* __restrict__ nvalid, TOut* __restrict__ y,
+                                       int S, int C, int tiles_per_row, int act_silu,
+                                       int residual) {
+    constexpr int R = TAPS - 1;
+    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (c >= C) return;
+    const int b = blockIdx.y / tiles_per_row;
+    const int t0 = (blockIdx.y % tiles_per_row) * SC_TT;
+    const int t1 = min(t0 + SC_TT, S);
+    const int slot = seq[b];
+    const int n = slot < 0 ? 0 : nvalid[b];
+    const int p0 = pos[(long)b * S];
+    float wr[8][TAPS];
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) wr[e][j] = w[(long)(c + e) * TAPS + j];
+    float hist[R > 0 ? R : 1][8];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int col = t0 - R + r;
+        if (col >= 0) {
+            load8<TIn>(x + ((long)b * S + col) * xs + c, hist[r]);
+        } else {
+            const float* tp = tail + ((long)(slot < 0 ? 0 : slot) * R + (R + col)) * C + c;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) hist[r][e] = (n > 0 && p0 + col >= 0) ? tp[e] : 0.f;
+        }
+    }
+    for (int t = t0; t < t1; ++t) {
+        float o[8];
+        if (t < n) {
+            float cur[8];
+            load8<TIn>(x + ((long)b * S + t) * xs + c, cur);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float acc = wr[e][R] * cur[e];
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc += wr[e][r] * hist[r][e];
+                if (act_silu) acc = acc * sigmoidf_(acc);
+                if (residual) acc += cur[e];
+                o[e] = acc;
+            }
+#pragma unroll
+            for (int r = 0; r + 1 < R; ++r)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) hist[r][e] = hist[r + 1][e];
+            if (R > 0) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) hist[R - 1][e] = cur[e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = 0.f;
+        }
+        TOut* yp = y + ((long)b * S + t) * C + c;
+        if constexpr (sizeof(TOut) == 2) {
+            uint32_t pk[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                uint32_t lo = __float_as_uint(o[2 * e]), hi = __float_as_uint(o[2 * e + 1]);
+                lo += 0x7fffu + ((lo >> 16) & 1u);
+                hi += 0x7fffu + ((hi >> 16) & 1u);
+                pk[e] = (lo >> 16) | (hi & 0xffff0000u);
+            }
+            *reinterpret_cast<uint4*>(yp) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        } else {
+            st8<float>(reinterpret_cast<float*>(yp), o);
+        }
+    }
+}
+
 // new tail = last R inputs of (old tail ++ this step's inputs); one thread per
 // (row, channel) so the in-place shift is private to the thread
 template <typename TIn>
@@ -183,25 +291,6 @@ __global__ void paged_kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc,
 // (NQ=4 rows, 16 waves) for pure decode steps, where one token's few heads
 // leave the key range as the only parallelism.
 #define ATT_NQ_MAX 16
-
-template <typename T> struct KVec8 { float v[8]; };
-
-template <typename T> DEV void load8(const T* p, float* v);
-template <> DEV void load8<bf16>(const bf16* p, float* v) {
-    const uint4 raw = *reinterpret_cast<const uint4*>(p);
-    const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        v[2 * e] = __uint_as_float(u[e] << 16);
-        v[2 * e + 1] = __uint_as_float(u[e] & 0xffff0000u);
-    }
-}
-template <> DEV void load8<float>(const float* p, float* v) {
-    const float4 a = *reinterpret_cast<const float4*>(p);
-    const float4 b = *reinterpret_cast<const float4*>(p + 4);
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-}
 
 template <typename T, typename TOut, int MAXR, int ATT_NQ, int ATT_WAVES>
 __global__ void __launch_bounds__(ATT_WAVES * WAVE)
@@ -947,10 +1036,32 @@ int nx_layer_norm(const float* x, const float* w, void* out, int out_bf16, long 
 }
 
 int nx_short_conv(const void* x, long xs, int x_bf16, const float* w, const float* tail,
-                  const int* pos, const int* seq, void* y, int y_bf16, int B, int S, int C,
-                  int taps, int act_silu, int residual, hipStream_t st) {
+                  const int* pos, const int* seq, const int* nvalid, void* y, int y_bf16, int B,
+                  int S, int C, int taps, int act_silu, int residual, hipStream_t st) {
     const long total = (long)B * S * C;
     if (total <= 0) return 0;
+    {
+        // tiled path: 8-channel groups with 16-byte accesses on every row
+        const int esz = x_bf16 ? 2 : 4;
+        const int tiles = (S + SC_TT - 1) / SC_TT;
+        const bool ok = taps >= 2 && taps <= 4 && (C % 8) == 0 && ((xs * esz) % 16) == 0 &&
+                        ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
+                        ((uintptr_t)tail % 16) == 0 && (long)B * tiles <= 65535 && S >= 8;
+        if (ok) {
+            dim3 gt((C / 8 + 127) / 128, (unsigned)(B * tiles)), bt(128);
+#define SCT(TI, TO, TP) short_conv_tile_kernel<TI, TO, TP><<<gt, bt, 0, st>>>( \
+        (const TI*)x, xs, w, tail, pos, seq, nvalid, (TO*)y, S, C, tiles, act_silu, residual)
+#define SCTT(TI, TO) do { if (taps == 2) SCT(TI, TO, 2); else if (taps == 3) SCT(TI, TO, 3); \
+                          else SCT(TI, TO, 4); } while (0)
+            if (x_bf16 && y_bf16) SCTT(bf16, bf16);
+            else if (x_bf16) SCTT(bf16, float);
+            else if (y_bf16) SCTT(float, bf16);
+            else SCTT(float, float);
+#undef SCTT
+#undef SCT
+            return (int)hipGetLastError();
+        }
+    }
     dim3 grid(grid_for(total, 256)), block(256);
 #define SC(TI, TO) short_conv_kernel<TI, TO><<<grid, block, 0, st>>>( \
         (const TI*)x, xs, w, tail, pos, seq, (TO*)y, B, S, C, taps, act_silu, residual)

@@ -149,7 +149,7 @@ def short_conv(x, w, tail, step: StepLayout, activation: str = "none",
         y = torch.empty(B, S, C, dtype=out_dtype, device=x.device)
         _check(lib.nx_short_conv(
             _p(x), ctypes.c_long(_rows_view(x)), _is_bf16(x), _p(_f32(w)), _p(tail), _p(step.positions),
-            _p(step.seq_ids), _p(y), _is_bf16(y), B, S, C, w.shape[1],
+            _p(step.seq_ids), _p(step.nvalid), _p(y), _is_bf16(y), B, S, C, w.shape[1],
             int(activation == "silu"), int(residual), _stream()), "short_conv")
         return y
     return ref.short_conv(x, w, tail, step.positions, step.seq_ids,

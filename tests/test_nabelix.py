@@ -195,11 +195,12 @@ def test_gelu_mul_and_residual_ops(device, ff):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("taps", [1, 2, 4])
 @pytest.mark.parametrize("act,residual", [("none", True), ("silu", False)])
-def test_short_conv_portions_and_slots(device, taps, act, residual):
+@pytest.mark.parametrize("C", [10, 16])               # per-element and 8-channel tiled kernels
+def test_short_conv_portions_and_slots(device, taps, act, residual, C):
     """Two sequences in different slots fed in unequal portions (down to one
     token) against the whole-sequence convolution."""
     torch.manual_seed(2)
-    C, T = 10, 17
+    T = 17
     conv = CausalShortConv(C, taps, activation=act, residual=residual)
     conv.weight.data = torch.randn(C, taps)
     conv = conv.to(device)
