@@ -82,6 +82,8 @@ def replay(engine, lines, out_dir: str, emit=print):
                 req = live.get(e["id"])
                 if req is None:
                     req = live[e["id"]] = engine.admit()
+                if not e.get("tokens"):
+                    continue                  # admitted, nothing to feed yet
                 parts.append((req, torch.tensor(e["tokens"], dtype=torch.long)))
                 wants.append(e.get("want", []))
             if parts:
