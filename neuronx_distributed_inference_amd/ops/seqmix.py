@@ -35,18 +35,41 @@ _lib_error: Optional[BaseException] = None
 _lock = threading.Lock()
 
 
+def _compile(dst: str) -> str:
+    hipcc = os.environ.get("HIPCC") or (
+        "/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else "hipcc")
+    tmp = dst + ".%d.tmp" % os.getpid()
+    try:
+        subprocess.run([hipcc] + HIPCC_FLAGS + ["-o", tmp, SRC_PATH], check=True,
+                       stdout=subprocess.DEVNULL, stderr=subprocess.PIPE)
+        os.replace(tmp, dst)
+    finally:
+        if os.path.exists(tmp):
+            os.unlink(tmp)
+    return dst
+
+
 def build(force: bool = False) -> str:
-    """Compile the library in-tree (cross-compiles without a GPU)."""
+    """Compile the library in-tree (cross-compiles without a GPU). When the
+    package directory is read-only the library goes to the user's temp
+    directory, named after the source's modification time."""
+    global LIB_PATH
     if not force and os.path.exists(LIB_PATH) and \
             os.path.getmtime(LIB_PATH) >= os.path.getmtime(SRC_PATH):
         return LIB_PATH
-    hipcc = os.environ.get("HIPCC") or (
-        "/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else "hipcc")
-    tmp = LIB_PATH + ".%d.tmp" % os.getpid()
-    subprocess.run([hipcc] + HIPCC_FLAGS + ["-o", tmp, SRC_PATH], check=True,
-                   stdout=subprocess.DEVNULL, stderr=subprocess.PIPE)
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    try:
+        return _compile(LIB_PATH)
+    except (OSError, subprocess.CalledProcessError):
+        if os.access(os.path.dirname(LIB_PATH), os.W_OK):
+            raise                      # a real compile error, not a read-only tree
+        import tempfile
+
+        alt = os.path.join(tempfile.gettempdir(), "nxdi_seqmix_%d_%d.so" % (
+            os.getuid(), int(os.path.getmtime(SRC_PATH))))
+        if force or not os.path.exists(alt):
+            _compile(alt)
+        LIB_PATH = alt
+        return LIB_PATH
 
 
 def _load():
