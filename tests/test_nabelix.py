@@ -312,6 +312,17 @@ def test_attention_other_shapes(device, L):
     _attention_alone(device, L, 23, [(22, 3), (12, 5)], page=8, cuts=[2, 7, 1, 13])
 
 
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cuts", [None, [100] + [1] * 50])
+def test_attention_far_keys_among_many(device, cuts):
+    """150 tokens: a kept first token 145 positions back, the first token
+    that is NOT kept, and the keys on both sides of the window's far edge,
+    each made to dominate its query's scores if the mask lets it."""
+    L = left_cfg(2, 1, 8, 8, size=40, keep=5, scale=0.5)
+    spikes = [(149, 4), (148, 5), (147, 108), (146, 106), (120, 0), (110, 70), (109, 70)]
+    _attention_alone(device, L, 150, spikes, page=16, cuts=cuts)
+
+
 @pytest.mark.gpu
 def test_attention_bf16_long_window_gpu():
     L = left_cfg(8, 2, 64, 128, size=200, keep=20, scale=0.1)
