@@ -142,7 +142,7 @@ class NabelixParallelMixer(nn.Module):
         H, G, Dk, Dv = lc["heads"], lc["kv_heads"], lc["dim"], lc["vdim"]
         self.splits = [H * Dk, G * Dk, G * Dv, H * Dv,        # left q k v gate
                        self.right.qkv_channels, rc["heads"],  # right q|k|v, beta
-                       self.decay_rank, self.gate_rank]
+                       self.decay_rank + self.gate_rank]      # low-rank first stages
         self.in_proj = ColumnParallelLinear(width, sum(self.splits), dtype=dtype, tp_degree=1)
         self.left_o = RowParallelLinear(H * Dv, width, dtype=dtype, tp_degree=1)
         self.right_o = RowParallelLinear(rc["heads"] * rc["vdim"], width, dtype=dtype,
@@ -150,9 +150,9 @@ class NabelixParallelMixer(nn.Module):
 
     def forward(self, h, kv_mgr, run_idx: int, step):
         y = self.in_proj(h)
-        lq, lk, lv, lg, rqkv, rb, ra, rg = torch.split(y, self.splits, dim=-1)
+        lq, lk, lv, lg, rqkv, rb, rag = torch.split(y, self.splits, dim=-1)
         left = self.left(lq, lk, lv, kv_mgr, run_idx, step, gate=lg)
-        right = self.right(rqkv, rb, ra, rg, kv_mgr.state, f"run{run_idx}", step)
+        right = self.right(rqkv, rb, rag, kv_mgr.state, f"run{run_idx}", step)
         return self.left_o(left), self.right_o(right)
 
 
@@ -318,8 +318,8 @@ class NabelixForCausalLM(CausalLMBase):
             out[d + "mixer.right_o.weight"] = w(R + "o")
             out[d + "mixer.right.conv.weight"] = torch.cat(
                 [f(R + "q.conv"), f(R + "k.conv"), f(R + "v.conv")], dim=0)
-            out[d + "mixer.right.a2.weight"] = w(R + "a2")
-            out[d + "mixer.right.g2.weight"] = w(R + "g2")
+            out[d + "mixer.right.ag2.weight"] = GatedDeltaRule.block_diagonal(
+                w(R + "a2"), w(R + "g2"))
             out[d + "mixer.right.A_log"] = f(R + "A_log")
             out[d + "mixer.right.dt_bias"] = f(R + "dt_bias")
             out[d + "mixer.right.norm_weight"] = f(R + "norm")

@@ -52,7 +52,7 @@ class DistanceBiasWindowAttention(nn.Module):
         kc, vc = kv_mgr.get_cache(cache_idx)
         k2 = k.reshape(B * S, k.shape[-1]) if k.is_contiguous() else k.flatten(0, 1)
         v2 = v.reshape(B * S, v.shape[-1]) if v.is_contiguous() else v.flatten(0, 1)
-        seqmix.paged_kv_write(kc.data, vc.data, k2, v2, kv_mgr.slot_mapping)
+        seqmix.paged_kv_write(kc.data, vc.data, k2, v2, kv_mgr.slot_mapping, step)
         return seqmix.window_bias_attention(
             q, kc.data, vc.data, step, kv_mgr.block_table, self.r1, self.r2,
             self.scale, self.window, self.keep_first, self.num_heads, gate=gate,

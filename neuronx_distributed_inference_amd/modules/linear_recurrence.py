@@ -42,10 +42,14 @@ class GatedDeltaRule(nn.Module):
         self.eps = float(eps)
         self.qkv_channels = 2 * num_kv_heads * dim + num_heads * vdim
         self.conv = CausalShortConv(self.qkv_channels, conv_taps, activation="silu")
-        self.a2 = ColumnParallelLinear(decay_rank, num_heads * dim, dtype=dtype,
-                                       tp_degree=tp_degree)
-        self.g2 = ColumnParallelLinear(gate_rank, num_heads * vdim, dtype=dtype,
-                                       tp_degree=tp_degree)
+        # second stages of the two low-rank projections as ONE block-diagonal
+        # GEMM: [a_low | g_low] (rank_a + rank_g) -> [a (H*dim) | gate (H*vdim)];
+        # the off-diagonal blocks are exact zeros
+        self.decay_rank = decay_rank
+        self.gate_rank = gate_rank
+        self.ag2 = ColumnParallelLinear(decay_rank + gate_rank,
+                                        num_heads * (dim + vdim), dtype=dtype,
+                                        tp_degree=tp_degree)
         f32 = dict(dtype=torch.float32)
         self.A_log = nn.Parameter(torch.zeros(num_heads, **f32), requires_grad=False)
         self.dt_bias = nn.Parameter(torch.zeros(num_heads * dim, **f32), requires_grad=False)
@@ -55,15 +59,23 @@ class GatedDeltaRule(nn.Module):
         return {"conv": self.conv.state_shape(),
                 "mem": (self.num_heads, self.vdim, self.dim)}   # stored transposed
 
-    def forward(self, qkv: torch.Tensor, beta: torch.Tensor, a_low: torch.Tensor,
-                g_low: torch.Tensor, states, key: str,
-                step: seqmix.StepLayout) -> torch.Tensor:
+    @staticmethod
+    def block_diagonal(a2: torch.Tensor, g2: torch.Tensor) -> torch.Tensor:
+        """(H*dim, rank_a), (H*vdim, rank_g) -> the fused second-stage weight."""
+        w = torch.zeros(a2.shape[0] + g2.shape[0], a2.shape[1] + g2.shape[1], dtype=a2.dtype)
+        w[:a2.shape[0], :a2.shape[1]] = a2
+        w[a2.shape[0]:, a2.shape[1]:] = g2
+        return w
+
+    def forward(self, qkv: torch.Tensor, beta: torch.Tensor, ag_low: torch.Tensor,
+                states, key: str, step: seqmix.StepLayout) -> torch.Tensor:
         """qkv (B,S,q|k|v channels) raw projections, beta (B,S,H) logits,
-        a_low / g_low the first-stage low-rank projections. `states` is the
-        RecurrentStateManager, `key` this layer run's prefix in it."""
+        ag_low (B,S,rank_a+rank_g) the first-stage low-rank projections
+        [decay | gate]. `states` is the RecurrentStateManager, `key` this
+        layer run's prefix in it."""
         qkv_c = self.conv(qkv, states.get(key + ".conv"), step, out_dtype=torch.float32)
-        a = self.a2(a_low)
-        gate = self.g2(g_low)
+        ag = self.ag2(ag_low)
+        a, gate = torch.split(ag, [self.num_heads * self.dim, self.num_heads * self.vdim], dim=-1)
         return seqmix.gated_delta_rule(
             qkv_c, beta, a, self.dt_bias, self.A_log, gate, self.norm_weight,
             self.eps, states.get(key + ".mem"), step, self.num_kv_heads, self.dim,

@@ -145,6 +145,16 @@ class StepLayout:
         self.positions = _i32(positions)
         self.seq_ids = _i32(seq_ids)
         self.nvalid = (self.positions >= 0).sum(-1).to(torch.int32)
+        self._i32 = {}
+
+    def i32(self, t: torch.Tensor) -> torch.Tensor:
+        """int32 copy of a per-step index tensor (block table, slot mapping),
+        converted once per step instead of once per layer."""
+        key = (t.data_ptr(), tuple(t.shape), t.dtype)
+        hit = self._i32.get(key)
+        if hit is None:
+            hit = self._i32[key] = (t, _i32(t))      # keeps `t` alive: the pointer stays its
+        return hit[1]
 
 
 # ----------------------------------------------------------------------
@@ -191,7 +201,7 @@ def short_conv_commit(x, tail, step: StepLayout):
     ref.short_conv_commit(x, tail, step.positions, step.seq_ids)
 
 
-def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping):
+def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping, step: "StepLayout" = None):
     """Scatter k_new (N, G*Dk) / v_new (N, G*Dv) rows (row-strided views
     allowed) into paged caches (blocks, block, G, D*)."""
     if k_cache.is_cuda:
@@ -205,7 +215,8 @@ def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping):
         _check(lib.nx_paged_kv_write(
             _p(k_cache), _p(v_cache), _p(k_new), ctypes.c_long(k_new.stride(0)),
             _p(v_new), ctypes.c_long(v_new.stride(0)), _is_bf16(k_cache),
-            _p(_i32(slot_mapping)), ctypes.c_long(N), GDk, GDv,
+            _p(_i32(slot_mapping) if step is None else step.i32(slot_mapping)),
+            ctypes.c_long(N), GDk, GDv,
             ctypes.c_long(k_cache.shape[0] * k_cache.shape[1]), _stream()),
             "paged_kv_write")
         return
@@ -227,7 +238,7 @@ def window_bias_attention(q, k_cache, v_cache, step: StepLayout, block_table,
     if q.is_cuda:
         lib = _load()
         out = torch.empty(B, S, H * Dv, dtype=out_dtype, device=q.device)
-        bt = _i32(block_table)
+        bt = step.i32(block_table)
         _check(lib.nx_window_attn(
             _p(q), ctypes.c_long(_rows_view(q)), _p(k_cache), _p(v_cache),
             _p(step.positions), _p(step.seq_ids), _p(bt), bt.shape[1],

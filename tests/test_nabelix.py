@@ -364,8 +364,7 @@ def _delta_alone(device, R, T, cuts, slots=(1,), eps=1e-4):
 
     mod = GatedDeltaRule(H, G, D, Dv, R["conv"], R["decay_rank"], R["gate_rank"], eps, F32)
     mod.conv.weight.data = torch.cat([W["p.q.conv"], W["p.k.conv"], W["p.v.conv"]]).float()
-    mod.a2.weight.data = W["p.a2"].float()
-    mod.g2.weight.data = W["p.g2"].float()
+    mod.ag2.weight.data = GatedDeltaRule.block_diagonal(W["p.a2"].float(), W["p.g2"].float())
     mod.A_log.data, mod.dt_bias.data = W["p.A_log"].float(), W["p.dt_bias"].float()
     mod.norm_weight.data = W["p.norm"].float()
     mod = mod.to(device)
@@ -377,14 +376,15 @@ def _delta_alone(device, R, T, cuts, slots=(1,), eps=1e-4):
     for t in mgr.state.tensors.values():        # dirty slots: a start must not read them
         t.data.normal_()
     qkv = torch.cat([h @ W["p.q"].T, h @ W["p.k"].T, h @ W["p.v"].T], 1).float()
-    beta, alow, glow = (h @ W["p.b"].T).float(), (h @ W["p.a1"].T).float(), (h @ W["p.g1"].T).float()
+    beta = (h @ W["p.b"].T).float()
+    aglow = torch.cat([h @ W["p.a1"].T, h @ W["p.g1"].T], 1).float()
     got, at = [], 0
     for n in cuts:
         sl = slice(at, at + n)
         pos = torch.arange(at, at + n).view(1, n).to(device)
         st = seqmix.StepLayout(pos, torch.tensor(list(slots)).to(device))
-        y = mod(qkv[sl][None].to(device), beta[sl][None].to(device), alow[sl][None].to(device),
-                glow[sl][None].to(device), mgr.state, "x", st)
+        y = mod(qkv[sl][None].to(device), beta[sl][None].to(device), aglow[sl][None].to(device),
+                mgr.state, "x", st)
         got.append(y[0].float().cpu())
         at += n
     close(torch.cat(got), want, 2e-4)
