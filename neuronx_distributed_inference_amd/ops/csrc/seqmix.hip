@@ -301,7 +301,9 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
                    const float* __restrict__ r2, const T* __restrict__ gate, long gstride,
                    TOut* __restrict__ out, int H, int G, int Dk, int Dv,
                    int bsz, int S, float scale, int window, int keep, int HPW, int QT,
-                   int chunks) {
+                   int chunks, int lpr, int pws) {
+    // lpr > 0 (decode shape only): P.V with 8 value channels per lane and
+    // 64/lpr keys per step, 16-byte V loads; pws = floats of LDS per wave
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int DkP = (Dk + 7) & ~7;                       // padded q row
     float* qs = smem;                                    // ATT_NQ * DkP
@@ -361,7 +363,13 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
 #pragma unroll
         for (int c = 0; c < MAXR; ++c) acc[r][c] = 0.f;
     }
-    float* myp = ps + wv * WAVE * ATT_NQ;
+    float* myp = ps + wv * pws;
+    constexpr int NV = ATT_NQ == 4 ? 8 : 1;
+    float acc8[ATT_NQ == 4 ? 4 : 1][NV];
+#pragma unroll
+    for (int r = 0; r < (ATT_NQ == 4 ? 4 : 1); ++r)
+#pragma unroll
+        for (int e = 0; e < NV; ++e) acc8[r][e] = 0.f;
 
     for (int rd = 0; rd < rounds; ++rd) {
         const int base = (rd * ATT_WAVES + wv) * WAVE;
@@ -422,6 +430,10 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
                 m_run[r] = m_new;
 #pragma unroll
                 for (int c = 0; c < MAXR; ++c) acc[r][c] *= corr;
+                if constexpr (ATT_NQ == 4) {
+#pragma unroll
+                    for (int e = 0; e < NV; ++e) acc8[r][e] *= corr;
+                }
                 sc[r] = p;
             }
 #pragma unroll
@@ -431,30 +443,79 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
         if (base < n) {
             const int cnt = min(WAVE, n - base);
             const int sl = (int)slot;
-            for (int mm = 0; mm < cnt; ++mm) {
-                const long sj = __shfl(sl, mm, WAVE);
-                const T* vp = vc + sj * vrow + (long)g * Dv;
-                float vv[MAXR];
+            bool done = false;
+            if constexpr (ATT_NQ == 4) {
+                if (lpr > 0) {
+                    done = true;
+                    const int ksub = WAVE / lpr;
+                    const int sub = lane / lpr, ch = (lane % lpr) * 8;
+                    for (int it = 0; it * ksub < cnt; ++it) {
+                        const int mm = it * ksub + sub;
+                        const long sj = __shfl(sl, mm < cnt ? mm : 0, WAVE);
+                        if (mm < cnt) {
+                            float vv[8];
+                            load8<T>(vc + sj * vrow + (long)g * Dv + ch, vv);
+                            const float4 pp = *reinterpret_cast<const float4*>(myp + mm * ATT_NQ);
 #pragma unroll
-                for (int c = 0; c < MAXR; ++c) {
-                    const int d = lane + c * WAVE;
-                    vv[c] = d < Dv ? ldf<T>(vp + d) : 0.f;
+                            for (int e = 0; e < 8; ++e) {
+                                acc8[0][e] += pp.x * vv[e];
+                                acc8[1][e] += pp.y * vv[e];
+                                acc8[2][e] += pp.z * vv[e];
+                                acc8[3][e] += pp.w * vv[e];
+                            }
+                        }
+                    }
                 }
-                const float4* p4 = reinterpret_cast<const float4*>(myp + mm * ATT_NQ);
-#pragma unroll
-                for (int r4 = 0; r4 < ATT_NQ / 4; ++r4) {
-                    const float4 pp = p4[r4];
+            }
+            if (!done) {
+                for (int mm = 0; mm < cnt; ++mm) {
+                    const long sj = __shfl(sl, mm, WAVE);
+                    const T* vp = vc + sj * vrow + (long)g * Dv;
+                    float vv[MAXR];
 #pragma unroll
                     for (int c = 0; c < MAXR; ++c) {
-                        acc[4 * r4][c] += pp.x * vv[c];
-                        acc[4 * r4 + 1][c] += pp.y * vv[c];
-                        acc[4 * r4 + 2][c] += pp.z * vv[c];
-                        acc[4 * r4 + 3][c] += pp.w * vv[c];
+                        const int d = lane + c * WAVE;
+                        vv[c] = d < Dv ? ldf<T>(vp + d) : 0.f;
+                    }
+                    const float4* p4 = reinterpret_cast<const float4*>(myp + mm * ATT_NQ);
+#pragma unroll
+                    for (int r4 = 0; r4 < ATT_NQ / 4; ++r4) {
+                        const float4 pp = p4[r4];
+#pragma unroll
+                        for (int c = 0; c < MAXR; ++c) {
+                            acc[4 * r4][c] += pp.x * vv[c];
+                            acc[4 * r4 + 1][c] += pp.y * vv[c];
+                            acc[4 * r4 + 2][c] += pp.z * vv[c];
+                            acc[4 * r4 + 3][c] += pp.w * vv[c];
+                        }
                     }
                 }
             }
         }
         __syncthreads();
+    }
+    if constexpr (ATT_NQ == 4) {
+        if (lpr > 0) {
+            // fold the key subgroups, then move to the channel-per-lane layout
+            // the merge and the epilogue use (through this wave's LDS region)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float v = acc8[r][e];
+                    for (int off = lpr; off < WAVE; off <<= 1) v += __shfl_xor(v, off, WAVE);
+                    if (lane < lpr) myp[r * Dv + lane * 8 + e] = v;
+                }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c = 0; c < MAXR; ++c) {
+                    const int d = lane + c * WAVE;
+                    if (d < Dv) acc[r][c] = myp[r * Dv + d];
+                }
+            __syncthreads();
+        }
     }
     // merge the waves' partial softmaxes pairwise (tree) through LDS
     for (int step = 1; step < ATT_WAVES; step <<= 1) {
@@ -1139,13 +1200,27 @@ int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, 
     const int chunks = (rep + HPW - 1) / HPW;
     const int DkP = (Dk + 7) & ~7;
     dim3 grid((S + QT - 1) / QT, G * chunks, B), block(NW * WAVE);
-    const long ptile = (long)NW * WAVE * NQ, marea = (long)(NW / 2) * NQ * (Dv + 2);
-    const size_t sh = (size_t)(NQ * DkP + (ptile > marea ? ptile : marea)) * sizeof(float);
+    // decode shape: 8 value channels per lane when they tile a wave evenly
+    int lpr = 0;
+    if (dec && (Dv % 8) == 0) {
+        const int l = Dv / 8;
+        if (l <= WAVE && (l & (l - 1)) == 0) lpr = l;
+    }
+    int pws = (lpr > 0 && NQ * Dv > WAVE * NQ) ? NQ * Dv : WAVE * NQ;
+    long ptile = (long)NW * pws;
+    const long marea = (long)(NW / 2) * NQ * (Dv + 2);
+    size_t sh = (size_t)(NQ * DkP + (ptile > marea ? ptile : marea)) * sizeof(float);
+    if (sh > 60 * 1024 && lpr > 0) {                      // wide values: scalar P.V
+        lpr = 0;
+        pws = WAVE * NQ;
+        ptile = (long)NW * pws;
+        sh = (size_t)(NQ * DkP + (ptile > marea ? ptile : marea)) * sizeof(float);
+    }
     if (sh > 60 * 1024) return -3;
 #define WA(T, TO, MR, Q, W) window_attn_kernel<T, TO, MR, Q, W><<<grid, block, sh, st>>>( \
         (const T*)q, qstride, (const T*)kc, (const T*)vc, pos, seq, btab, max_blocks, r1, r2, \
         (const T*)gate, gstride, (TO*)out, H, G, Dk, Dv, bsz, S, scale, window, keep, HPW, QT, \
-        chunks)
+        chunks, lpr, pws)
 #define WAS(T, TO, MR) do { if (dec) WA(T, TO, MR, 4, 16); else WA(T, TO, MR, 16, 4); } while (0)
 #define WAM(T, TO) do { if (Dv <= 2 * WAVE) WAS(T, TO, 2); else WAS(T, TO, 4); } while (0)
     if (io_bf16 && out_bf16) WAM(bf16, bf16);
