@@ -100,10 +100,29 @@ class NabelixInferenceConfig(InferenceConfig):
             from safetensors import safe_open
 
             with safe_open(ckpt, framework="pt") as st:
+                names = set(st.keys())
+
+                def shape(name):
+                    return st.get_slice(name).get_shape() if name in names else None
+
+                emb = shape("embed")
+                if emb:
+                    hf.setdefault("vocab", emb[0])
+                    hf.setdefault("width", emb[1])
+                c0 = shape("l0.canon1")
+                if c0 and not hf.get("canon"):
+                    hf["canon"] = {"taps": c0[1]}
                 for i, lc in enumerate(hf["layers"]):
                     rc = lc["mixer"]["right"]
-                    rc["decay_rank"] = st.get_slice(f"l{i}.mix.right.a1").get_shape()[0]
-                    rc["gate_rank"] = st.get_slice(f"l{i}.mix.right.g1").get_shape()[0]
+                    rc["decay_rank"] = shape(f"l{i}.mix.right.a1")[0]
+                    rc["gate_rank"] = shape(f"l{i}.mix.right.g1")[0]
+                    # sizes the file may leave to the tensors
+                    cv = shape(f"l{i}.mix.right.q.conv")
+                    if cv and "conv" not in rc:
+                        rc["conv"] = cv[1]
+                    gate = shape(f"l{i}.mlp.gate")
+                    if gate and isinstance(lc.get("mlp"), dict) and "ff" not in lc["mlp"]:
+                        lc["mlp"]["ff"] = gate[0]
         return cls(neuron_config=neuron_config, **hf)
 
     def run_order(self) -> List[int]:
