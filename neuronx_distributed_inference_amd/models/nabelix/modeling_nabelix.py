@@ -36,7 +36,8 @@ import torch
 import torch.nn as nn
 
 from neuronx_distributed_inference_amd.config import InferenceConfig
-from neuronx_distributed_inference_amd.models.model_base import CausalLMBase, DecoderModel
+from neuronx_distributed_inference_amd.models.hybrid_base import HybridDecoderModel
+from neuronx_distributed_inference_amd.models.model_base import CausalLMBase
 from neuronx_distributed_inference_amd.modules.attention.distance_bias import (
     DistanceBiasWindowAttention,
 )
@@ -193,6 +194,9 @@ class NabelixLayer(nn.Module):
                                 hidden_act="gelu_pytorch_tanh", fused_gate_up=True)
             self.mlp.act_mul_fused = seqmix.gelu_tanh_mul_fused
 
+    def kv_shape(self):
+        return self.mixer.left.kv_shape()
+
     def state_shapes(self) -> Dict[str, tuple]:
         out = {"canon": self.canon.state_shape()}
         out.update(self.mixer.right.state_shapes())
@@ -211,19 +215,6 @@ class NabelixLayer(nn.Module):
         return x
 
 
-class _LayerRun:
-    """One execution of a layer against its own cache/state index, with the
-    engine's layer-call signature."""
-
-    def __init__(self, layer: NabelixLayer, run_idx: int):
-        self.layer = layer
-        self.run_idx = run_idx
-
-    def __call__(self, h, residual, cos, sin, kv_mgr, position_ids, phase,
-                 attention_mask, seq_ids, **_):
-        return self.layer(h, kv_mgr, self.run_idx), None
-
-
 class _FinalNorm(LayerNorm):
     def __init__(self, width, eps, out_dtype):
         super().__init__(width, eps=eps)
@@ -233,64 +224,16 @@ class _FinalNorm(LayerNorm):
         return seqmix.layer_norm(x, self.weight, self.eps, self.out_dtype)
 
 
-class NabelixModel(DecoderModel):
-    def build_rotary(self, config):
-        return None
-
+class NabelixModel(HybridDecoderModel):
     def build_layers(self, config) -> nn.ModuleList:
         return nn.ModuleList(NabelixLayer(config, i) for i in range(len(config.layers)))
 
     def build_norm(self, config) -> nn.Module:
         return _FinalNorm(config.width, config.norm["eps"], config.neuron_config.torch_dtype)
 
-    def build_kv_manager(self, config) -> nn.Module:
-        from neuronx_distributed_inference_amd.modules.kvcache.block_kv_cache_manager import (
-            BlockKVCacheManager,
-        )
-
-        ec = config.neuron_config
-        self._order = config.run_order()
+    def run_order(self, config):
         self._pass_starts = set(config.pass_starts())
-        self._runs = [(li, _LayerRun(self.layers[li], ri)) for ri, li in enumerate(self._order)]
-        self.max_blocks_per_seq = (ec.max_length + ec.pa_block_size - 1) // ec.pa_block_size
-        num_blocks = ec.pa_num_blocks or self.max_blocks_per_seq * ec.kv_cache_batch_size
-        mgr = BlockKVCacheManager(
-            num_layers=len(self._order), num_kv_heads=1, head_dim=1,
-            num_blocks=num_blocks, block_size=ec.pa_block_size, dtype=ec.torch_dtype,
-            tp_degree=1,
-            layer_kv_shapes=[self.layers[li].mixer.left.kv_shape() for li in self._order],
-            state_slots=ec.kv_cache_batch_size,
-        )
-        for ri, li in enumerate(self._order):
-            for name, shape in self.layers[li].state_shapes().items():
-                mgr.state.register(f"run{ri}.{name}", shape)
-        return mgr
-
-    # -- engine hooks ---------------------------------------------------
-    def begin_step(self, position_ids, seq_ids, block_table):
-        B = position_ids.shape[0]
-        if seq_ids is None:
-            seq_ids = torch.arange(B, device=position_ids.device)
-        self.kv_mgr.step = seqmix.StepLayout(position_ids, seq_ids)
-        if block_table is None:
-            # callers without a page table (plain generate loops) get the
-            # linear layout: slot s owns pages [s*M, (s+1)*M)
-            M = self.max_blocks_per_seq
-            if self.kv_mgr.num_blocks < self.kv_mgr.state.num_slots * M:
-                raise RuntimeError(
-                    "the page pool is smaller than slots x max_length: pass a block_table")
-            sid = seq_ids.long().view(B, 1)
-            block_table = torch.where(
-                sid >= 0,
-                sid * M + torch.arange(M, device=position_ids.device).view(1, M),
-                torch.full_like(sid, -1))     # pad rows own no pages
-        return block_table
-
-    def prepare_hidden(self, h):
-        return h.float()
-
-    def layer_runs(self):
-        return self._runs
+        return config.run_order()
 
     def before_layer_run(self, run_idx, h, h_embed):
         if run_idx == 0:

@@ -1,0 +1,92 @@
+"""Latent (low-rank KV) attention with a softmax sink.
+
+Each token stores only a normed latent ``c`` (``kv_rank`` channels) and one
+rotated key part shared by all heads (``rot_dim`` channels). Per head the
+unrotated key is ``W_uk c`` and the value ``W_uv c``; the score is
+``(q_plain . k_plain + q_rot . k_rot) * scale``. Rotary positions use the
+interleaved pair layout on the first ``rot_dims`` channels of the rotated
+part. The softmax denominator carries one extra term ``exp(sink_h)`` per
+head: a key without a value, unscaled.
+
+The engine computes this in the *absorbed* form, which never expands the
+cache: ``q_plain . (W_uk c) = (W_uk^T q_plain) . c``, so the query is mapped
+into latent space (one small batched GEMM per step), attention runs as
+multi-query attention over cache rows ``[c | k_rot]`` whose values are the
+rows' own first ``kv_rank`` channels, and ``W_uv`` is applied to the
+attended latent afterwards. One page row per token holds everything; there
+is no value cache.
+
+The module owns the latent norm, the two up-projections, the sink and the
+cache access; the projections of the layer input (queries and the
+down-projection) are the caller's.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from neuronx_distributed_inference_amd.modules.norm import StreamRMSNorm
+from neuronx_distributed_inference_amd.modules.rope import interleaved_inv_freq
+from neuronx_distributed_inference_amd.ops import seqmix
+
+
+class LatentSinkAttention(nn.Module):
+    def __init__(self, num_heads: int, dim: int, rot_dim: int, v_dim: int, kv_rank: int,
+                 scale: float, eps: float, rope_base: float, rot_dims: int,
+                 dtype: torch.dtype, sink: bool = True):
+        super().__init__()
+        assert rot_dims <= rot_dim and rot_dims % 2 == 0
+        self.num_heads = num_heads
+        self.dim = dim
+        self.rot_dim = rot_dim
+        self.v_dim = v_dim
+        self.kv_rank = kv_rank
+        self.scale = float(scale)
+        self.row = kv_rank + rot_dim                      # one cache row
+        self.latent_norm = StreamRMSNorm(kv_rank, eps=eps, one_plus=False)
+        self.register_buffer("inv_freq", interleaved_inv_freq(rope_base, rot_dims),
+                             persistent=False)
+        # per-head up-projections, stored for the batched products:
+        # uk (H, dim, kv_rank): q_plain -> latent space;  uv_t (H, kv_rank, v_dim)
+        self.uk = nn.Parameter(torch.zeros(num_heads, dim, kv_rank, dtype=dtype),
+                               requires_grad=False)
+        self.uv_t = nn.Parameter(torch.zeros(num_heads, kv_rank, v_dim, dtype=dtype),
+                                 requires_grad=False)
+        self.sink = nn.Parameter(torch.zeros(num_heads, dtype=torch.float32),
+                                 requires_grad=False) if sink else None
+
+    def kv_shape(self):
+        """One key 'head' of kv_rank + rot_dim channels, no value pages."""
+        return (1, self.row, 0)
+
+    def forward(self, q: torch.Tensor, dkv: torch.Tensor, kv_mgr, cache_idx: int,
+                step: seqmix.StepLayout) -> torch.Tensor:
+        """q (B,S,H*(dim+rot_dim)), dkv (B,S,kv_rank+rot_dim): column slices
+        of a fused projection are fine. Returns (B,S,H*v_dim)."""
+        B, S = q.shape[0], q.shape[1]
+        H, D, R, C = self.num_heads, self.dim, self.rot_dim, self.kv_rank
+        T = B * S
+        dt = q.dtype
+        # cache row [rms_norm(latent) | rotated shared key part]
+        row = torch.empty(B, S, self.row, dtype=dt, device=q.device)
+        self.latent_norm(dkv[..., :C], out=row[..., :C])
+        seqmix.rotate_interleaved(dkv[..., C:].unsqueeze(2), step, self.inv_freq,
+                                  out=row[..., C:].unsqueeze(2))
+        kc, _ = kv_mgr.get_cache(cache_idx)
+        seqmix.paged_kv_write(kc.data, None, row.view(T, self.row), None,
+                              kv_mgr.slot_mapping, step)
+        # query in latent space: [uk_h^T q_plain | rotated q_rot] per head
+        q4 = q.view(B, S, H, D + R) if q.is_contiguous() else q.unflatten(-1, (H, D + R))
+        qa = torch.empty(B, S, H, self.row, dtype=dt, device=q.device)
+        torch.bmm(q4[..., :D].flatten(0, 1).transpose(0, 1), self.uk,
+                  out=qa.view(T, H, self.row)[..., :C].transpose(0, 1))
+        seqmix.rotate_interleaved(q4[..., D:], step, self.inv_freq, out=qa[..., C:])
+        k_cache = kc.data
+        lat = seqmix.paged_attention(
+            qa.view(B, S, H * self.row), k_cache, k_cache[..., :C], step, kv_mgr.block_table,
+            self.scale, H, sink=self.sink, out_dtype=dt)              # (B,S,H*C)
+        out = torch.empty(B, S, H * self.v_dim, dtype=dt, device=q.device)
+        torch.bmm(lat.view(T, H, C).transpose(0, 1), self.uv_t,
+                  out=out.view(T, H, self.v_dim).transpose(0, 1))
+        return out

@@ -29,12 +29,18 @@ class BlockKVCacheManager(nn.Module):
         block_size: int = 128,
         dtype: torch.dtype = torch.bfloat16,
         tp_degree: Optional[int] = None,
-        layer_kv_shapes: Optional[List[Tuple[int, int, int]]] = None,
+        layer_kv_shapes: Optional[List[Optional[Tuple[int, int, int]]]] = None,
         state_slots: int = 0,
+        layer_kv_source: Optional[List[Optional[int]]] = None,
     ):
         """`layer_kv_shapes`: optional per-layer (kv_heads, k_head_dim,
         v_head_dim) for models whose layers differ or whose keys and values
-        have different head sizes; overrides num_kv_heads/head_dim.
+        have different head sizes; overrides num_kv_heads/head_dim. An entry
+        of None is a layer without pages of its own (a recurrent layer, or
+        one that reads another layer's pages: `layer_kv_source[i]` names the
+        lender and `get_cache(i)` returns its tensors); v_head_dim 0 is a
+        layer whose values are channels of its key rows (latent caches): it
+        gets key pages only.
         `state_slots` > 0 attaches a :class:`RecurrentStateManager` as
         ``self.state`` for models that also carry fixed-size per-sequence
         state (linear recurrences, short-convolution tails)."""
@@ -49,17 +55,23 @@ class BlockKVCacheManager(nn.Module):
         if layer_kv_shapes is None:
             layer_kv_shapes = [(num_kv_heads, head_dim, head_dim)] * num_layers
         assert len(layer_kv_shapes) == num_layers
-        self.layer_kv_shapes = [(max(g // tp, 1), dk, dv) for g, dk, dv in layer_kv_shapes]
+        self.layer_kv_shapes = [None if sh is None else (max(sh[0] // tp, 1), sh[1], sh[2])
+                                for sh in layer_kv_shapes]
+        self.layer_kv_source = list(layer_kv_source or [None] * num_layers)
+        for i, src in enumerate(self.layer_kv_source):
+            if src is not None:
+                assert self.layer_kv_shapes[i] is None and self.layer_kv_shapes[src] is not None, \
+                    "a borrowing layer owns no pages and its lender does"
+
+        def pages(sh, which):
+            if sh is None or sh[which] == 0:
+                return torch.zeros(0, dtype=dtype)          # placeholder: no pages
+            return torch.zeros((num_blocks, block_size, sh[0], sh[which]), dtype=dtype)
+
         self.k_caches = nn.ParameterList(
-            nn.Parameter(torch.zeros((num_blocks, block_size, g, dk), dtype=dtype),
-                         requires_grad=False)
-            for g, dk, _ in self.layer_kv_shapes
-        )
+            nn.Parameter(pages(sh, 1), requires_grad=False) for sh in self.layer_kv_shapes)
         self.v_caches = nn.ParameterList(
-            nn.Parameter(torch.zeros((num_blocks, block_size, g, dv), dtype=dtype),
-                         requires_grad=False)
-            for g, _, dv in self.layer_kv_shapes
-        )
+            nn.Parameter(pages(sh, 2), requires_grad=False) for sh in self.layer_kv_shapes)
         self.state = RecurrentStateManager(state_slots) if state_slots > 0 else None
 
     @property
@@ -67,7 +79,8 @@ class BlockKVCacheManager(nn.Module):
         return self.state is not None
 
     def estimate_bytes(self) -> int:
-        return sum(k.numel() * k.element_size() * 2 for k in self.k_caches)
+        return sum(t.numel() * t.element_size() for c in (self.k_caches, self.v_caches)
+                   for t in c)
 
     # per-forward step context set by DecoderModel (block table + slots)
     def set_step_context(self, block_table: torch.Tensor, slot_mapping: torch.Tensor):
@@ -83,6 +96,9 @@ class BlockKVCacheManager(nn.Module):
         return self._slot_mapping
 
     def get_cache(self, layer_idx: int, bucket_len=None):
+        src = self.layer_kv_source[layer_idx]
+        if src is not None:
+            layer_idx = src
         return self.k_caches[layer_idx], self.v_caches[layer_idx]
 
     def update_cache(self, layer_idx: int, k_new, v_new, positions, seq_ids=None):

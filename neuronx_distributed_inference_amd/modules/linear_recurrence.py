@@ -7,11 +7,14 @@ Per head the state is a (dim x vdim) fp32 matrix ``M`` updated once per token
     M <- M + k_t u^T
     o_t = M^T q_t                                (reads the fresh write)
 
-with one decay per head AND key channel, unit-norm q/k (q also scaled by
-dim^-1/2), beta a sigmoid. q/k/v first pass a short causal convolution and
-SiLU; the output is RMS-normalised per head, scaled by a weight shared
-across heads and multiplied by a sigmoid gate. ``a_t`` and the gate come
-through low-rank two-stage projections whose second stages live here.
+with one decay per head AND key channel (``decay_per_channel``) or a single
+one per head, unit-norm q/k (q also scaled by dim^-1/2), beta a sigmoid.
+q/k/v first pass a short causal convolution and SiLU; the output is
+RMS-normalised per head, scaled by a weight shared across heads and
+multiplied by a gate (``gate_act``: sigmoid or silu of the gate projection).
+``a_t`` and the gate either come through low-rank two-stage projections whose
+second stages live here (``decay_rank``/``gate_rank`` > 0) or are handed in
+at full size by the caller (ranks 0).
 
 State (``M`` and the convolution tail) is engine state in the cache
 manager's :class:`RecurrentStateManager`, keyed by this module's name and
@@ -32,9 +35,14 @@ from neuronx_distributed_inference_amd.parallel.layers import ColumnParallelLine
 class GatedDeltaRule(nn.Module):
     def __init__(self, num_heads: int, num_kv_heads: int, dim: int, vdim: int,
                  conv_taps: int, decay_rank: int, gate_rank: int, eps: float,
-                 dtype: torch.dtype, tp_degree: int = 1):
+                 dtype: torch.dtype, tp_degree: int = 1,
+                 decay_per_channel: bool = True, gate_act: str = "sigmoid"):
         super().__init__()
         assert num_heads % num_kv_heads == 0
+        assert (decay_rank > 0) == (gate_rank > 0), "both low-rank or both direct"
+        assert gate_act in ("sigmoid", "silu")
+        self.decay_per_channel = bool(decay_per_channel)
+        self.gate_act = gate_act
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads
         self.dim = dim
@@ -47,12 +55,15 @@ class GatedDeltaRule(nn.Module):
         # the off-diagonal blocks are exact zeros
         self.decay_rank = decay_rank
         self.gate_rank = gate_rank
-        self.ag2 = ColumnParallelLinear(decay_rank + gate_rank,
-                                        num_heads * (dim + vdim), dtype=dtype,
-                                        tp_degree=tp_degree)
+        self.decay_width = num_heads * (dim if decay_per_channel else 1)
+        self.ag2 = None
+        if decay_rank > 0:
+            self.ag2 = ColumnParallelLinear(decay_rank + gate_rank,
+                                            self.decay_width + num_heads * vdim, dtype=dtype,
+                                            tp_degree=tp_degree)
         f32 = dict(dtype=torch.float32)
         self.A_log = nn.Parameter(torch.zeros(num_heads, **f32), requires_grad=False)
-        self.dt_bias = nn.Parameter(torch.zeros(num_heads * dim, **f32), requires_grad=False)
+        self.dt_bias = nn.Parameter(torch.zeros(self.decay_width, **f32), requires_grad=False)
         self.norm_weight = nn.Parameter(torch.ones(vdim, **f32), requires_grad=False)
 
     def state_shapes(self):
@@ -68,15 +79,21 @@ class GatedDeltaRule(nn.Module):
         return w
 
     def forward(self, qkv: torch.Tensor, beta: torch.Tensor, ag_low: torch.Tensor,
-                states, key: str, step: seqmix.StepLayout) -> torch.Tensor:
-        """qkv (B,S,q|k|v channels) raw projections, beta (B,S,H) logits,
-        ag_low (B,S,rank_a+rank_g) the first-stage low-rank projections
-        [decay | gate]. `states` is the RecurrentStateManager, `key` this
-        layer run's prefix in it."""
+                states, key: str, step: seqmix.StepLayout,
+                gate: torch.Tensor = None) -> torch.Tensor:
+        """qkv (B,S,q|k|v channels) raw projections, beta (B,S,H) logits.
+        With low-rank stages: ag_low (B,S,rank_a+rank_g), the first-stage
+        projections [decay | gate]. Without: ag_low is the decay projection
+        itself (B,S,decay_width) and ``gate`` (B,S,H*vdim) the gate's.
+        `states` is the RecurrentStateManager, `key` this layer run's prefix
+        in it."""
         qkv_c = self.conv(qkv, states.get(key + ".conv"), step, out_dtype=torch.float32)
-        ag = self.ag2(ag_low)
-        a, gate = torch.split(ag, [self.num_heads * self.dim, self.num_heads * self.vdim], dim=-1)
+        if self.ag2 is not None:
+            ag = self.ag2(ag_low)
+            a, gate = torch.split(ag, [self.decay_width, self.num_heads * self.vdim], dim=-1)
+        else:
+            a = ag_low
         return seqmix.gated_delta_rule(
             qkv_c, beta, a, self.dt_bias, self.A_log, gate, self.norm_weight,
             self.eps, states.get(key + ".mem"), step, self.num_kv_heads, self.dim,
-            self.vdim, out_dtype=a.dtype)
+            self.vdim, out_dtype=a.dtype, gate_act=self.gate_act)

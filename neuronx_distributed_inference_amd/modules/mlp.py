@@ -29,6 +29,8 @@ class GatedMLP(nn.Module):
         bias: bool = False,
         group=None,
         fused_gate_up: bool = False,
+        act_limit: float = 7.0,
+        act_alpha: float = 1.702,
     ):
         super().__init__()
         self.fused = fused_gate_up
@@ -72,6 +74,14 @@ class GatedMLP(nn.Module):
         elif hidden_act in ("gelu", "gelu_pytorch_tanh", "gelu_new"):
             self.act_mul = ops.gelu_tanh_mul
             self.act_mul_fused = ops.gelu_tanh_mul_fused
+        elif hidden_act == "clamped_swiglu":
+            # g = min(gate, limit), u = clamp(up, +-limit):
+            # g * sigmoid(alpha * g) * (u + 1); limit and alpha are parameters
+            from neuronx_distributed_inference_amd.ops import ref, seqmix
+
+            lim, al = float(act_limit), float(act_alpha)
+            self.act_mul = lambda g, u: ref.clamped_glu(g, u, lim, al).to(g.dtype)
+            self.act_mul_fused = lambda gu: seqmix.clamped_glu_fused(gu, lim, al)
         else:
             raise ValueError(f"unsupported hidden_act {hidden_act}")
 

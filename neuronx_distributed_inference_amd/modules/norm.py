@@ -59,3 +59,33 @@ class LayerNorm(nn.Module):
         if residual is None:
             return xf
         return xf, new_res
+
+
+class StreamRMSNorm(nn.Module):
+    """RMS norm for models whose residual stream is fp32: statistics and the
+    weight product in fp32, output in the dtype the consumer asks for.
+    ``one_plus`` selects weights stored around zero (scale = 1 + w). Besides
+    the plain call, :meth:`add_into` does the post-norm residual step
+    ``stream += norm(y)`` in one kernel and hands back the updated stream in
+    the next GEMM's input dtype."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-6, one_plus: bool = False,
+                 out_dtype: torch.dtype = torch.float32):
+        super().__init__()
+        init = torch.zeros if one_plus else torch.ones
+        self.weight = nn.Parameter(init(hidden_size, dtype=torch.float32), requires_grad=False)
+        self.eps = float(eps)
+        self.one_plus = bool(one_plus)
+        self.out_dtype = out_dtype
+
+    def forward(self, x: torch.Tensor, residual: torch.Tensor = None, out=None):
+        from neuronx_distributed_inference_amd.ops import seqmix
+
+        assert residual is None
+        return seqmix.rms_norm(x, self.weight, self.eps, self.one_plus,
+                               out_dtype=None if out is not None else self.out_dtype, out=out)
+
+    def add_into(self, stream: torch.Tensor, y: torch.Tensor, copy_dtype=None):
+        from neuronx_distributed_inference_amd.ops import seqmix
+
+        return seqmix.add_rms_norm(stream, y, self.weight, self.eps, self.one_plus, copy_dtype)

@@ -153,3 +153,11 @@ def rope_apply_interleaved(q: torch.Tensor, k: torch.Tensor,
     q_out = torch.stack([q1 * c - q2 * s, q2 * c + q1 * s], dim=-1).flatten(-2)
     k_out = torch.stack([k1 * c - k2 * s, k2 * c + k1 * s], dim=-1).flatten(-2)
     return q_out.to(q.dtype), k_out.to(k.dtype)
+
+
+def interleaved_inv_freq(base: float, dims: int) -> torch.Tensor:
+    """Frequencies base^(-2i/dims), i < dims/2, for rotary layouts that pair
+    channel 2i with 2i+1. Evaluated in float64 and rounded once, so the fp32
+    table is the closest one to the exact values."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float()

@@ -291,18 +291,25 @@ def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping):
     ok = slot_mapping >= 0
     idx = slot_mapping[ok].long()
     kc = k_cache.view(-1, *k_cache.shape[2:])
-    vc = v_cache.view(-1, *v_cache.shape[2:])
     kc[idx] = k_new[ok].to(kc.dtype)
-    vc[idx] = v_new[ok].to(vc.dtype)
+    if v_cache is not None:          # caches whose values live inside the key rows
+        vc = v_cache.view(-1, *v_cache.shape[2:])
+        vc[idx] = v_new[ok].to(vc.dtype)
 
 
-def window_bias_attention(q, k_cache, v_cache, positions, block_table, r1, r2,
-                          scale, window, keep_first, gate=None,
-                          out_dtype=torch.float32):
-    """Softmax attention of ragged queries against a paged cache. Query at
-    position i sees key j <= i when i-j < window or j < keep_first; the
-    score is q.k*scale - r1_h*log1p(r2_h*(i-j)). q (B,S,H,Dk) ->
-    (B,S,H*Dv), optionally multiplied by sigmoid(gate)."""
+def paged_attention(q, k_cache, v_cache, positions, block_table, scale,
+                    window=None, keep_first=0, r1=None, r2=None, gate=None,
+                    softcap=0.0, sink=None, q_temp=None, out_dtype=torch.float32):
+    """Softmax attention of ragged queries against a paged cache, every
+    option a parameter. Query at position i sees key j <= i when no window
+    is given, else when i-j < window or j < keep_first. Score, in order:
+    q.k * scale * temp(i) with temp(i) = 1 + coef*ln(floor((i+1)/every)+1)
+    (``q_temp`` = (coef, every)); minus r1_h*log1p(r2_h*(i-j)) when r1/r2
+    are given; then softcap*tanh(score/softcap) when softcap > 0. ``sink``
+    (H,) adds exp(sink_h) to the softmax denominator (a key without value).
+    ``v_cache`` may be a narrowed view of ``k_cache`` (values stored inside
+    the key rows). q (B,S,H,Dk) -> (B,S,H*Dv), optionally times
+    sigmoid(gate)."""
     B, S, H, Dk = q.shape
     G, Dv = v_cache.shape[2], v_cache.shape[3]
     bs = k_cache.shape[1]
@@ -319,12 +326,24 @@ def window_bias_attention(q, k_cache, v_cache, positions, block_table, r1, r2,
         s = torch.einsum("bshd,blhd->bhsl", q.float(), k) * scale
         i = positions.view(B, 1, S, 1).float()
         j = torch.arange(L, device=q.device).view(1, 1, 1, L).float()
-        dist = (i - j).clamp(min=0)
-        s = s - r1.float().view(1, H, 1, 1) * torch.log1p(
-            r2.float().view(1, H, 1, 1) * dist)
-        vis = (j <= i) & ((i - j < window) | (j < keep_first))
+        if q_temp is not None:
+            coef, every = q_temp
+            s = s * (1.0 + coef * torch.log(torch.floor((i.clamp(min=0) + 1) / every) + 1.0))
+        if r1 is not None:
+            dist = (i - j).clamp(min=0)
+            s = s - r1.float().view(1, H, 1, 1) * torch.log1p(
+                r2.float().view(1, H, 1, 1) * dist)
+        if softcap:
+            s = softcap * torch.tanh(s / softcap)
+        vis = j <= i
+        if window is not None:
+            vis = vis & ((i - j < window) | (j < keep_first))
         s = s.masked_fill(~vis, float("-inf"))
-        p = torch.nan_to_num(torch.softmax(s, dim=-1))
+        if sink is not None:
+            sk = sink.float().view(1, H, 1, 1).expand(B, H, S, 1)
+            p = torch.nan_to_num(torch.softmax(torch.cat([s, sk], -1), dim=-1))[..., :L]
+        else:
+            p = torch.nan_to_num(torch.softmax(s, dim=-1))
         out = torch.einsum("bhsl,blhd->bshd", p, v)
     out = out.reshape(B, S, H * Dv)
     if gate is not None:
@@ -332,16 +351,26 @@ def window_bias_attention(q, k_cache, v_cache, positions, block_table, r1, r2,
     return out.to(out_dtype)
 
 
+def window_bias_attention(q, k_cache, v_cache, positions, block_table, r1, r2,
+                          scale, window, keep_first, gate=None,
+                          out_dtype=torch.float32):
+    """Sliding window plus kept first tokens, log-distance score penalty."""
+    return paged_attention(q, k_cache, v_cache, positions, block_table, scale,
+                           window=window, keep_first=keep_first, r1=r1, r2=r2,
+                           gate=gate, out_dtype=out_dtype)
+
+
 def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps, state,
                      positions, seq_ids, kv_heads, dim, vdim,
-                     out_dtype=torch.float32):
-    """Delta-rule recurrence with a per-key-channel decay, carried state
+                     out_dtype=torch.float32, gate_act="sigmoid"):
+    """Delta-rule recurrence with a decay per head and key channel (``a``
+    (B,S,H*dim)) or one per head (``a`` (B,S,H), dt_bias (H)), carried state
     (slots, H, vdim, dim) fp32 (stored transposed: a value channel's key
     rows are contiguous). qkv (B,S,2*G*dim + H*vdim) holds the
     convolved+activated q|k|v; beta (B,S,H) and a (B,S,H*dim), gate
     (B,S,H*vdim) are pre-activation projections. Per token and head:
       S <- diag(decay) S ; u = beta (v - S^T k) ; S <- S + k u^T ; o = S^T q
-    followed by o / rms(o) * norm_w * sigmoid(gate)."""
+    followed by o / rms(o) * norm_w * act(gate), act = sigmoid or silu."""
     B, S, _ = qkv.shape
     G, D, Dv = kv_heads, dim, vdim
     H = beta.shape[-1]
@@ -355,8 +384,8 @@ def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps, state,
     q = q.repeat_interleave(rep, dim=2)
     k = k.repeat_interleave(rep, dim=2)
     bt = torch.sigmoid(beta.float())
-    dt = torch.nn.functional.softplus(a.float() + dt_bias.float()).view(B, S, H, D)
-    decay = torch.exp(-torch.exp(a_log.float()).view(1, 1, H, 1) * dt)
+    dt = torch.nn.functional.softplus(a.float() + dt_bias.float()).view(B, S, H, -1)
+    decay = torch.exp(-torch.exp(a_log.float()).view(1, 1, H, 1) * dt).expand(B, S, H, D)
     out = torch.zeros(B, S, H, Dv, dtype=torch.float32, device=qkv.device)
     n_valid, p0s = _row_extent(positions)
     for b in range(B):
@@ -373,9 +402,45 @@ def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps, state,
             out[b, t] = torch.einsum("hdv,hd->hv", St, q[b, t])
         state[slot] = St.transpose(-1, -2).to(state.dtype)
     out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps) * norm_w.float()
-    out = out.reshape(B, S, H * Dv) * torch.sigmoid(gate.float())
+    gf = gate.float()
+    gf = torch.sigmoid(gf) if gate_act == "sigmoid" else torch.nn.functional.silu(gf)
+    out = out.reshape(B, S, H * Dv) * gf
     return out.to(out_dtype)
 
 
 def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
     return cap * torch.tanh(logits.float() / cap)
+
+
+def rms_norm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float,
+                  one_plus: bool, out_dtype: torch.dtype) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) * w  (or * (1 + w)), fp32 statistics."""
+    xf = x.float()
+    w = weight.float()
+    y = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps) * (1.0 + w if one_plus else w)
+    return y.to(out_dtype)
+
+
+def rotate_interleaved(x: torch.Tensor, positions: torch.Tensor,
+                       inv_freq: torch.Tensor) -> torch.Tensor:
+    """Rotary positions on channel pairs (2i, 2i+1) of the first
+    2*len(inv_freq) channels of the last axis, angle p * inv_freq[i] in
+    fp32; the other channels pass unchanged. x (B,S,N,C), positions (B,S);
+    returns fp32."""
+    B, S = positions.shape
+    dims = 2 * inv_freq.numel()
+    xf = x.float().clone()
+    ang = positions.clamp(min=0).float().view(B, S, 1, 1) * inv_freq.float()
+    c, sn = torch.cos(ang), torch.sin(ang)
+    a, b = xf[..., 0:dims:2].clone(), xf[..., 1:dims:2].clone()
+    xf[..., 0:dims:2] = a * c - b * sn
+    xf[..., 1:dims:2] = b * c + a * sn
+    return xf
+
+
+def clamped_glu(gate: torch.Tensor, up: torch.Tensor, limit: float,
+                alpha: float = 1.702) -> torch.Tensor:
+    """min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, +-limit) + 1)."""
+    g = gate.float().clamp(max=limit)
+    u = up.float().clamp(-limit, limit)
+    return g * torch.sigmoid(alpha * g) * (u + 1.0)

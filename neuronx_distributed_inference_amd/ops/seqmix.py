@@ -146,6 +146,9 @@ class StepLayout:
         self.seq_ids = _i32(seq_ids)
         self.nvalid = (self.positions >= 0).sum(-1).to(torch.int32)
         self._i32 = {}
+        # the residual stream in the GEMM input dtype, handed from one
+        # sublayer's residual kernel to the next sublayer (None: not yet made)
+        self.stream_copy = None
 
     def i32(self, t: torch.Tensor) -> torch.Tensor:
         """int32 copy of a per-step index tensor (block table, slot mapping),
@@ -203,18 +206,22 @@ def short_conv_commit(x, tail, step: StepLayout):
 
 def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping, step: "StepLayout" = None):
     """Scatter k_new (N, G*Dk) / v_new (N, G*Dv) rows (row-strided views
-    allowed) into paged caches (blocks, block, G, D*)."""
+    allowed) into paged caches (blocks, block, G, D*). ``v_cache``/``v_new``
+    may be None for caches whose values live inside the key rows."""
     if k_cache.is_cuda:
         lib = _load()
         N = k_new.shape[0]
         GDk = k_cache.shape[2] * k_cache.shape[3]
-        GDv = v_cache.shape[2] * v_cache.shape[3]
-        assert k_new.shape[1] == GDk and v_new.shape[1] == GDv
-        assert k_new.dtype == k_cache.dtype == v_new.dtype == v_cache.dtype
-        assert k_new.stride(1) == 1 and v_new.stride(1) == 1
+        GDv = 0 if v_cache is None else v_cache.shape[2] * v_cache.shape[3]
+        assert k_new.shape[1] == GDk and k_new.dtype == k_cache.dtype and k_new.stride(1) == 1
+        assert k_cache.is_contiguous()
+        if v_cache is not None:
+            assert v_new.shape[1] == GDv and v_new.dtype == v_cache.dtype == k_cache.dtype
+            assert v_new.stride(1) == 1 and v_cache.is_contiguous()
         _check(lib.nx_paged_kv_write(
             _p(k_cache), _p(v_cache), _p(k_new), ctypes.c_long(k_new.stride(0)),
-            _p(v_new), ctypes.c_long(v_new.stride(0)), _is_bf16(k_cache),
+            _p(v_new), ctypes.c_long(0 if v_new is None else v_new.stride(0)),
+            _is_bf16(k_cache),
             _p(_i32(slot_mapping) if step is None else step.i32(slot_mapping)),
             ctypes.c_long(N), GDk, GDv,
             ctypes.c_long(k_cache.shape[0] * k_cache.shape[1]), _stream()),
@@ -222,14 +229,20 @@ def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping, step: "StepLayo
         return
     G = k_cache.shape[2]
     ref.paged_kv_write(k_cache, v_cache, k_new.reshape(k_new.shape[0], G, -1),
-                       v_new.reshape(v_new.shape[0], G, -1), slot_mapping)
+                       None if v_new is None else v_new.reshape(v_new.shape[0], G, -1),
+                       slot_mapping)
 
 
-def window_bias_attention(q, k_cache, v_cache, step: StepLayout, block_table,
-                          r1, r2, scale: float, window: int, keep_first: int,
-                          num_heads: int, gate=None, out_dtype=None):
+def paged_attention(q, k_cache, v_cache, step: StepLayout, block_table, scale: float,
+                    num_heads: int, window: Optional[int] = None, keep_first: int = 0,
+                    r1=None, r2=None, gate=None, softcap: float = 0.0, sink=None,
+                    q_temp=None, out_dtype=None):
     """q (B,S,H*Dk) (row-strided view allowed) against the paged cache ->
-    (B,S,H*Dv); see ref.window_bias_attention for the masking and bias."""
+    (B,S,H*Dv). Options (see ref.paged_attention): sliding ``window`` with
+    ``keep_first`` always-visible tokens (None = plain causal), log-distance
+    penalty ``r1``/``r2``, tanh score cap, per-head softmax ``sink``, query
+    temperature ``q_temp`` = (coef, every), sigmoid output ``gate``.
+    ``v_cache`` may be ``k_cache[..., :Dv]`` (values inside the key rows)."""
     B, S = q.shape[0], q.shape[1]
     H = num_heads
     G, Dk = k_cache.shape[2], k_cache.shape[3]
@@ -239,29 +252,55 @@ def window_bias_attention(q, k_cache, v_cache, step: StepLayout, block_table,
         lib = _load()
         out = torch.empty(B, S, H * Dv, dtype=out_dtype, device=q.device)
         bt = step.i32(block_table)
-        _check(lib.nx_window_attn(
-            _p(q), ctypes.c_long(_rows_view(q)), _p(k_cache), _p(v_cache),
+        assert k_cache.stride(3) == 1 and v_cache.stride(3) == 1
+        assert k_cache.stride(1) == k_cache.stride(2) * G and v_cache.stride(1) == v_cache.stride(2) * G
+        assert k_cache.stride(0) == k_cache.stride(1) * k_cache.shape[1]
+        assert v_cache.stride(0) == v_cache.stride(1) * v_cache.shape[1]
+        assert k_cache.dtype == v_cache.dtype == q.dtype
+        coef, every = (0.0, 0) if q_temp is None else (float(q_temp[0]), int(q_temp[1]))
+        _check(lib.nx_paged_attn(
+            _p(q), ctypes.c_long(_rows_view(q)), _p(k_cache), ctypes.c_long(k_cache.stride(1)),
+            ctypes.c_long(k_cache.stride(2)), _p(v_cache), ctypes.c_long(v_cache.stride(1)),
+            ctypes.c_long(v_cache.stride(2)),
             _p(step.positions), _p(step.seq_ids), _p(bt), bt.shape[1],
-            _p(_f32(r1)), _p(_f32(r2)),
+            _p(None if r1 is None else _f32(r1)), _p(None if r2 is None else _f32(r2)),
+            _p(None if sink is None else _f32(sink)),
             _p(gate), ctypes.c_long(0 if gate is None else _rows_view(gate)),
             _p(out), _is_bf16(q), _is_bf16(out), B, S, H, G, Dk, Dv,
-            k_cache.shape[1], ctypes.c_float(scale), int(window), int(keep_first),
-            _stream()), "window_bias_attention")
+            k_cache.shape[1], ctypes.c_float(scale),
+            int(window) if window is not None else 0x7fffffff, int(keep_first),
+            ctypes.c_float(softcap or 0.0), ctypes.c_float(coef), every,
+            _stream()), "paged_attention")
         return out
-    return ref.window_bias_attention(
-        q.reshape(B, S, H, Dk), k_cache, v_cache, step.positions, block_table,
-        r1, r2, scale, window, keep_first, gate=gate, out_dtype=out_dtype)
+    return ref.paged_attention(
+        q.reshape(B, S, H, Dk), k_cache, v_cache, step.positions, block_table, scale,
+        window=window, keep_first=keep_first, r1=r1, r2=r2, gate=gate,
+        softcap=softcap or 0.0, sink=sink, q_temp=q_temp, out_dtype=out_dtype)
+
+
+def window_bias_attention(q, k_cache, v_cache, step: StepLayout, block_table,
+                          r1, r2, scale: float, window: int, keep_first: int,
+                          num_heads: int, gate=None, out_dtype=None):
+    """Sliding window + kept first tokens with a log-distance penalty."""
+    return paged_attention(q, k_cache, v_cache, step, block_table, scale, num_heads,
+                           window=window, keep_first=keep_first, r1=r1, r2=r2,
+                           gate=gate, out_dtype=out_dtype)
 
 
 def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps: float,
                      state, step: StepLayout, kv_heads: int, dim: int, vdim: int,
-                     out_dtype=torch.float32):
+                     out_dtype=torch.float32, gate_act: str = "sigmoid"):
     """Gated delta-rule recurrence over the step's tokens, state carried in
-    `state` (slots, H, vdim, dim) fp32; see ref.gated_delta_rule."""
+    `state` (slots, H, vdim, dim) fp32; see ref.gated_delta_rule. ``a`` is
+    (B,S,H*dim) for a decay per key channel or (B,S,H) for one per head."""
+    assert gate_act in ("sigmoid", "silu")
     if qkv.is_cuda:
         lib = _load()
         B, S = qkv.shape[0], qkv.shape[1]
         H = beta.shape[-1]
+        per_head = a.shape[-1] == H and dim != 1
+        assert a.shape[-1] == (H if per_head else H * dim)
+        assert dt_bias.numel() == a.shape[-1]
         assert qkv.dtype == torch.float32 and state.dtype == torch.float32
         assert beta.dtype == a.dtype == gate.dtype == out_dtype
         out = torch.empty(B, S, H * vdim, dtype=out_dtype, device=qkv.device)
@@ -275,12 +314,13 @@ def gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps: float,
             _p(_f32(a_log)), _p(_f32(norm_w)), ctypes.c_float(eps), _p(state),
             _p(step.positions), _p(step.seq_ids), _p(step.nvalid), _p(prep),
             ctypes.c_long(PS), _p(obuf), _p(out),
-            _is_bf16(beta), B, S, H, kv_heads, dim, vdim, _stream()),
+            _is_bf16(beta), B, S, H, kv_heads, dim, vdim, int(per_head),
+            int(gate_act == "silu"), _stream()),
             "gated_delta_rule")
         return out
     return ref.gated_delta_rule(qkv, beta, a, dt_bias, a_log, gate, norm_w, eps,
                                 state, step.positions, step.seq_ids, kv_heads,
-                                dim, vdim, out_dtype)
+                                dim, vdim, out_dtype, gate_act)
 
 
 def softcap(logits, cap: float):
@@ -327,3 +367,101 @@ def gelu_tanh_mul_fused(gate_up):
         return out
     g, u = gate_up.float().chunk(2, dim=-1)
     return ref.gelu_tanh_mul(g, u).to(gate_up.dtype)
+
+
+def rms_norm(x, weight, eps: float, one_plus: bool = False, out_dtype=None, out=None):
+    """RMS norm over the last axis with fp32 statistics: x / sqrt(mean(x^2)
+    + eps) * w (or * (1 + w) for weights stored around zero). ``x`` may be a
+    column slice of a wider tensor; ``out`` may be a column slice to fill."""
+    out_dtype = out_dtype or (out.dtype if out is not None else x.dtype)
+    if x.is_cuda:
+        lib = _load()
+        C = x.shape[-1]
+        if out is None:
+            out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        assert out.shape == x.shape and out.dtype == out_dtype
+        rows = x.numel() // C
+        _check(lib.nx_rms_norm(
+            _p(x), ctypes.c_long(_rows_view(x)), _is_bf16(x), _p(_f32(weight)), int(one_plus),
+            ctypes.c_float(eps), _p(out), ctypes.c_long(_rows_view(out)), _is_bf16(out),
+            ctypes.c_long(rows), C, _stream()), "rms_norm")
+        return out
+    y = ref.rms_norm_rows(x, weight, eps, one_plus, out_dtype)
+    if out is not None:
+        out.copy_(y)
+        return out
+    return y
+
+
+def add_rms_norm(stream, y, weight, eps: float, one_plus: bool = True, copy_dtype=None):
+    """Post-norm residual step on the fp32 stream, in place:
+    stream += rms_norm(y) * (1 + w). Returns the updated stream cast to
+    ``copy_dtype`` (the next sublayer's GEMM input) or None."""
+    if stream.is_cuda:
+        lib = _load()
+        assert stream.dtype == torch.float32 and stream.is_contiguous()
+        y = y.contiguous()
+        C = stream.shape[-1]
+        copy = None
+        if copy_dtype is not None and copy_dtype != torch.float32:
+            copy = torch.empty(stream.shape, dtype=copy_dtype, device=stream.device)
+        _check(lib.nx_add_rms_norm(
+            _p(stream), _p(y), _is_bf16(y), _p(_f32(weight)), int(one_plus),
+            ctypes.c_float(eps), _p(copy), ctypes.c_long(stream.numel() // C), C,
+            _stream()), "add_rms_norm")
+        if copy_dtype == torch.float32:
+            return stream
+        return copy
+    stream.add_(ref.rms_norm_rows(y, weight, eps, one_plus, torch.float32))
+    if copy_dtype is None:
+        return None
+    return stream if copy_dtype == torch.float32 else stream.to(copy_dtype)
+
+
+def rotate_interleaved(x, step: StepLayout, inv_freq, out=None, out_dtype=None):
+    """Rotary positions on interleaved channel pairs (2i, 2i+1) of the first
+    2*len(inv_freq) channels of every head; angles p * inv_freq[i] in fp32.
+    x (B,S,N,C), possibly a strided view; ``out`` likewise (may be a slice of
+    a wider buffer). Channels past the rotated ones are copied."""
+    out_dtype = out_dtype or (out.dtype if out is not None else x.dtype)
+    if x.is_cuda:
+        lib = _load()
+        B, S, N, C = x.shape
+        if out is None:
+            out = torch.empty(B, S, N, C, dtype=out_dtype, device=x.device)
+        for t in (x, out):
+            assert t.stride(3) == 1 and t.stride(0) == t.stride(1) * S
+        assert 2 * inv_freq.numel() <= C
+        _check(lib.nx_rope_pairs(
+            _p(x), ctypes.c_long(x.stride(1)), ctypes.c_long(x.stride(2)), _is_bf16(x),
+            _p(out), ctypes.c_long(out.stride(1)), ctypes.c_long(out.stride(2)), _is_bf16(out),
+            _p(step.positions), _p(_f32(inv_freq)), inv_freq.numel(),
+            ctypes.c_long(B * S), N, C, _stream()), "rotate_interleaved")
+        return out
+    y = ref.rotate_interleaved(x, step.positions, inv_freq).to(out_dtype)
+    if out is not None:
+        out.copy_(y)
+        return out
+    return y
+
+
+def clamped_glu_fused(gate_up, limit: float, alpha: float = 1.702):
+    """(rows, 2I) [gate | up] -> g*sigmoid(alpha*g)*(u+1) with g = min(gate,
+    limit), u = clamp(up, -limit, limit)."""
+    I = gate_up.shape[-1] // 2
+    if gate_up.is_cuda:
+        lib = _load()
+        gu = gate_up.contiguous()
+        out = torch.empty(gu.shape[:-1] + (I,), dtype=gu.dtype, device=gu.device)
+        _check(lib.nx_clamped_glu(_p(gu), _p(out), _is_bf16(gu),
+                                  ctypes.c_long(gu.numel() // (2 * I)), I,
+                                  ctypes.c_float(limit), ctypes.c_float(alpha), _stream()),
+               "clamped_glu_fused")
+        return out
+    g, u = gate_up.chunk(2, dim=-1)
+    return ref.clamped_glu(g, u, limit, alpha).to(gate_up.dtype)
+
+
+def scaled_embedding(h, scale: float):
+    """Embedding rows -> fp32 residual stream, times a constant."""
+    return h.float().mul_(scale) if h.dtype != torch.float32 else h * scale

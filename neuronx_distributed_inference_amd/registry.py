@@ -71,6 +71,11 @@ _REGISTRY: Dict[str, Tuple[str, str, str]] = {
         "NabelixInferenceConfig",
         "NabelixForCausalLM",
     ),
+    "soputar": (
+        "neuronx_distributed_inference_amd.models.soputar.modeling_soputar",
+        "SoputarInferenceConfig",
+        "SoputarForCausalLM",
+    ),
     # conditional-generation families (multimodal / speech): resolved for
     # programmatic use; the CLI's causal-lm run path does not drive these
     "whisper": (
