@@ -60,6 +60,7 @@ class LatentSinkAttention(nn.Module):
         """One key 'head' of kv_rank + rot_dim channels, no value pages."""
         return (1, self.row, 0)
 
+    @torch.no_grad()           # inference only: the batched products write into views
     def forward(self, q: torch.Tensor, dkv: torch.Tensor, kv_mgr, cache_idx: int,
                 step: seqmix.StepLayout) -> torch.Tensor:
         """q (B,S,H*(dim+rot_dim)), dkv (B,S,kv_rank+rot_dim): column slices
@@ -77,7 +78,7 @@ class LatentSinkAttention(nn.Module):
         seqmix.paged_kv_write(kc.data, None, row.view(T, self.row), None,
                               kv_mgr.slot_mapping, step)
         # query in latent space: [uk_h^T q_plain | rotated q_rot] per head
-        q4 = q.view(B, S, H, D + R) if q.is_contiguous() else q.unflatten(-1, (H, D + R))
+        q4 = q.unflatten(-1, (H, D + R))
         qa = torch.empty(B, S, H, self.row, dtype=dt, device=q.device)
         torch.bmm(q4[..., :D].flatten(0, 1).transpose(0, 1), self.uk,
                   out=qa.view(T, H, self.row)[..., :C].transpose(0, 1))

@@ -1,8 +1,10 @@
-// Sequence-mixing kernels for hybrid models (gfx950): bias-free LayerNorm on
-// an fp32 residual stream, short causal convolutions with a carried tail,
-// paged KV scatter with distinct K/V head sizes, windowed softmax attention
-// with a log-distance penalty and always-visible first tokens, and the gated
-// delta-rule linear recurrence.
+// Sequence-mixing kernels for hybrid models (gfx950): bias-free LayerNorm and
+// RMS norms on an fp32 residual stream (with the post-norm residual step fused),
+// short causal convolutions with a carried tail, paged KV scatter with distinct
+// K/V head sizes, interleaved rotary positions, paged softmax attention with
+// optional sliding window / always-visible first tokens / log-distance penalty /
+// query temperature / tanh score cap / softmax sink, the gated delta-rule
+// linear recurrence, and gated feed-forward activations.
 //
 // Built as a plain C-ABI shared library (no torch headers): the Python side
 // passes raw device pointers and the current HIP stream, so the kernels are
@@ -272,11 +274,18 @@ __global__ void paged_kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc,
         const int s = slots[tok];
         if (s < 0 || s >= nslots) continue;
         if (e < GDk) kc[(long)s * GDk + e] = k[tok * kstride + e];
-        else vc[(long)s * GDv + (e - GDk)] = v[tok * vstride + (e - GDk)];
+        else vc[(long)s * GDv + (e - GDk)] = v[tok * vstride + (e - GDk)];   // GDv = 0: no V
     }
 }
 
-// ------------------------------------------------- windowed biased attention
+// ----------------------------------------------------------- paged attention
+// Score of query i and key j, in order: q.k * scale * temp(i), temp(i) = 1 +
+// qt_coef * ln(floor((i+1)/qt_every) + 1) (qt_every = 0: none); minus
+// r1_h * log(1 + r2_h (i-j)) (r1 = null: none); cap * tanh(. / cap) (cap = 0:
+// none). Visible: j <= i and (i-j < window or j < keep); plain causal attention
+// passes window = INT_MAX. `sink` (per head, or null) adds exp(sink_h) to the
+// softmax denominator. K and V rows are addressed as slot*tok_stride +
+// head*head_stride, so V may be a channel range of the K rows.
 // Workgroup (4 waves) = ATT_NQ query rows that share one KV head: HPW query
 // heads of the group x QT consecutive tokens of a batch row, so every K/V
 // line fetched serves all of them. The union of the rows' visible keys is
@@ -301,7 +310,9 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
                    const float* __restrict__ r2, const T* __restrict__ gate, long gstride,
                    TOut* __restrict__ out, int H, int G, int Dk, int Dv,
                    int bsz, int S, float scale, int window, int keep, int HPW, int QT,
-                   int chunks, int lpr, int pws) {
+                   int chunks, int lpr, int pws, long ktok, long khead, long vtok, long vhead,
+                   int kvec, const float* __restrict__ sink, float cap, float qt_coef,
+                   int qt_every) {
     // lpr > 0 (decode shape only): P.V with 8 value channels per lane and
     // 64/lpr keys per step, 16-byte V loads; pws = floats of LDS per wave
     extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -311,7 +322,7 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
     float* cs = ps;                                      // merge area reuses the P tiles
     constexpr int ATT_THREADS = ATT_WAVES * WAVE;
     __shared__ int rpos[ATT_NQ_MAX];
-    __shared__ float ra1[ATT_NQ_MAX], ra2[ATT_NQ_MAX];
+    __shared__ float ra1[ATT_NQ_MAX], ra2[ATT_NQ_MAX], rtemp[ATT_NQ_MAX], rsink[ATT_NQ_MAX];
 
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wv = tid / WAVE;
     const int b = blockIdx.z;
@@ -326,8 +337,11 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
         if (tq < QT && t0 + tq < S && hh < rep) p = pos[(long)b * S + t0 + tq];
         rpos[tid] = p;
         const int h = g * rep + (hh < rep ? hh : 0);
-        ra1[tid] = r1[h];
-        ra2[tid] = r2[h];
+        ra1[tid] = r1 ? r1[h] : 0.f;
+        ra2[tid] = r1 ? r2[h] : 0.f;
+        rsink[tid] = sink ? sink[h] : -INFINITY;
+        rtemp[tid] = (qt_every > 0 && p >= 0)
+            ? 1.f + qt_coef * logf((float)((p + 1) / qt_every) + 1.f) : 1.f;
     }
     __syncthreads();
     int i_min = 0x7fffffff, i_max = -1;
@@ -343,7 +357,7 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
         float v = 0.f;
         if (rpos[r] >= 0 && d < Dk) {
             const int tq = r / HPW, h = g * rep + chunk * HPW + r % HPW;
-            v = ldf<T>(q + ((long)b * S + t0 + tq) * qstride + (long)h * Dk + d) * scale;
+            v = ldf<T>(q + ((long)b * S + t0 + tq) * qstride + (long)h * Dk + d) * (scale * rtemp[r]);
         }
         qs[idx] = v;
     }
@@ -355,7 +369,6 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
     const int n = nfirst + (i_max - lo + 1);
     const int ntiles = (n + WAVE - 1) / WAVE;
     const int rounds = (ntiles + ATT_WAVES - 1) / ATT_WAVES;
-    const long krow = (long)G * Dk, vrow = (long)G * Dv;
     float m_run[ATT_NQ], l_run[ATT_NQ], acc[ATT_NQ][MAXR];
 #pragma unroll
     for (int r = 0; r < ATT_NQ; ++r) {
@@ -386,8 +399,8 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
                 const int blk = bt[j / bsz];
                 slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
             }
-            const T* kp = kc + slot * krow + (long)g * Dk;
-            if ((Dk & 7) == 0) {
+            const T* kp = kc + slot * ktok + (long)g * khead;
+            if (kvec) {
                 for (int d = 0; d < Dk; d += 8) {
                     float kv[8];
                     load8<T>(kp + d, kv);
@@ -416,9 +429,13 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
                 const bool vis = kvalid && dist >= 0 && (dist < window || j < keep);
                 float sv = -INFINITY;
                 if (vis) {
-                    const float x = ra2[r] * (float)dist;
-                    const float lg = sizeof(T) == 4 ? log1pf(x) : __logf(1.f + x);
-                    sv = sc[r] - ra1[r] * lg;
+                    sv = sc[r];
+                    if (r1) {                            // uniform
+                        const float x = ra2[r] * (float)dist;
+                        const float lg = sizeof(T) == 4 ? log1pf(x) : __logf(1.f + x);
+                        sv -= ra1[r] * lg;
+                    }
+                    if (cap > 0.f) sv = cap * tanhf(sv / cap);
                 }
                 const float m_new = fmaxf(m_run[r], wave_max(sv));
                 float p = 0.f, corr = 1.f;
@@ -454,7 +471,7 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
                         const long sj = __shfl(sl, mm < cnt ? mm : 0, WAVE);
                         if (mm < cnt) {
                             float vv[8];
-                            load8<T>(vc + sj * vrow + (long)g * Dv + ch, vv);
+                            load8<T>(vc + sj * vtok + (long)g * vhead + ch, vv);
                             const float4 pp = *reinterpret_cast<const float4*>(myp + mm * ATT_NQ);
 #pragma unroll
                             for (int e = 0; e < 8; ++e) {
@@ -470,7 +487,7 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
             if (!done) {
                 for (int mm = 0; mm < cnt; ++mm) {
                     const long sj = __shfl(sl, mm, WAVE);
-                    const T* vp = vc + sj * vrow + (long)g * Dv;
+                    const T* vp = vc + sj * vtok + (long)g * vhead;
                     float vv[MAXR];
 #pragma unroll
                     for (int c = 0; c < MAXR; ++c) {
@@ -558,7 +575,12 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
         if (rpos[r] < 0) continue;
         const int tq = r / HPW, h = g * rep + chunk * HPW + r % HPW;
         const long tok = (long)b * S + t0 + tq;
-        const float inv = 1.f / l_run[r];
+        float inv = 1.f / l_run[r];
+        if (sink) {                                      // one more term in the denominator
+            const float mf = fmaxf(m_run[r], rsink[r]);
+            const float ca = expf(m_run[r] - mf);
+            inv = ca / (l_run[r] * ca + expf(rsink[r] - mf));
+        }
         TOut* op = out + (tok * H + h) * (long)Dv;
         const T* gp = gate ? gate + tok * gstride + (long)h * Dv : nullptr;
 #pragma unroll
@@ -573,15 +595,17 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
     }
 }
 
-// ------------------------------------- windowed biased attention, matrix cores
-// bf16 prompt-portion path. Workgroup = 64 query rows of one KV head (4 waves x
-// 16 rows: the group's heads x consecutive tokens); all waves walk the same
-// 64-key tiles, staged once in LDS (K row-major, V transposed). Scores are
-// computed transposed, S^T = K Q^T (mfma 16x16x32 bf16, fp32 accumulate), so a
-// lane ends up with 16 scores of ONE query row and the probabilities already
-// sit in the A-operand layout of the P.V product. Bias, mask and online softmax
-// are fp32 per lane; P enters the second product as a hi + lo bf16 pair (16
-// mantissa bits), V as stored.
+// -------------------------------------------------- paged attention, matrix cores
+// bf16 prompt-portion path, same scores and options as above. Workgroup = 64
+// query rows of one KV head (4 waves x 16 rows: the group's heads x consecutive
+// tokens); all waves walk the same 64-key tiles, staged once in LDS (K row-major,
+// V transposed). Scores are computed transposed, S^T = K Q^T (mfma 16x16x32 bf16,
+// fp32 accumulate), so a lane ends up with 16 scores of ONE query row and the
+// probabilities already sit in the A-operand layout of the P.V product. Scale,
+// temperature, bias, cap, mask and online softmax are fp32 per lane; P enters the
+// second product as a hi + lo bf16 pair (16 mantissa bits), V as stored.
+// DKP / DVP are the head sizes padded to multiples of 32; the true Dk, Dv (any
+// multiples of 8) come at run time and the padding is zero-filled in LDS.
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 #define MA_ROWS 64
@@ -593,21 +617,23 @@ DEV uint16_t f2bf_rne(float f) {
     return (uint16_t)(u >> 16);
 }
 
-template <int DK, int DV>
+template <int DKP, int DVP>
 __global__ void __launch_bounds__(256)
-window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __restrict__ kc,
-                        const bf16* __restrict__ vc, const int* __restrict__ pos,
-                        const int* __restrict__ seq, const int* __restrict__ btab,
-                        int max_blocks, const float* __restrict__ r1,
-                        const float* __restrict__ r2, const bf16* __restrict__ gate,
-                        long gstride, bf16* __restrict__ out, int H, int G, int bsz, int S,
-                        float scale, int window, int keep, int QT) {
-    constexpr int KS = DK + 8;               // K tile row stride (elements)
+paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __restrict__ kc,
+                       const bf16* __restrict__ vc, const int* __restrict__ pos,
+                       const int* __restrict__ seq, const int* __restrict__ btab,
+                       int max_blocks, const float* __restrict__ r1,
+                       const float* __restrict__ r2, const bf16* __restrict__ gate,
+                       long gstride, bf16* __restrict__ out, int H, int G, int Dk, int Dv,
+                       int bsz, int S, float scale, int window, int keep, int QT, long ktok,
+                       long khead, long vtok, long vhead, const float* __restrict__ sink,
+                       float cap, float qt_coef, int qt_every) {
+    constexpr int KS = DKP + 8;              // K tile row stride (elements)
     constexpr int VS = MA_KT + 8;            // V^T tile row stride
     __shared__ __attribute__((aligned(16))) uint16_t k_lds[MA_KT * KS];
-    __shared__ __attribute__((aligned(16))) uint16_t vt_lds[DV * VS];
+    __shared__ __attribute__((aligned(16))) uint16_t vt_lds[DVP * VS];
     __shared__ int rpos[MA_ROWS];
-    __shared__ float ra1[MA_ROWS], ra2[MA_ROWS];
+    __shared__ float ra1[MA_ROWS], ra2[MA_ROWS], rsink[MA_ROWS];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int lr = lane & 15, lg = lane >> 4;
     const int b = blockIdx.z, g = blockIdx.y, t0 = blockIdx.x * QT;
@@ -616,8 +642,9 @@ window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __
     if (tid < MA_ROWS) {
         const int tq = tid / rep, hh = tid % rep;
         rpos[tid] = (tq < QT && t0 + tq < S) ? pos[(long)b * S + t0 + tq] : -1;
-        ra1[tid] = r1[g * rep + hh];
-        ra2[tid] = r2[g * rep + hh];
+        ra1[tid] = r1 ? r1[g * rep + hh] : 0.f;
+        ra2[tid] = r1 ? r2[g * rep + hh] : 0.f;
+        rsink[tid] = sink ? sink[g * rep + hh] : -INFINITY;
     }
     __syncthreads();
     int i_min = 0x7fffffff, i_max = -1;
@@ -630,14 +657,17 @@ window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __
     const int myrow = wv * 16 + lr;
     const int my_i = rpos[myrow];
     const float a1 = ra1[myrow], a2 = ra2[myrow];
-    bf16x8_t qf[DK / 32];
+    const float qscale = (qt_every > 0 && my_i >= 0)
+        ? scale * (1.f + qt_coef * logf((float)((my_i + 1) / qt_every) + 1.f)) : scale;
+    bf16x8_t qf[DKP / 32];
     {
         const int tq = myrow / rep, h = g * rep + myrow % rep;
-        const bf16* qp = q + ((long)b * S + t0 + tq) * qstride + (long)h * DK;
+        const bf16* qp = q + ((long)b * S + t0 + tq) * qstride + (long)h * Dk;
 #pragma unroll
-        for (int ks = 0; ks < DK / 32; ++ks) {
+        for (int ks = 0; ks < DKP / 32; ++ks) {
             uint4 raw = make_uint4(0, 0, 0, 0);
-            if (my_i >= 0) raw = *reinterpret_cast<const uint4*>(qp + ks * 32 + lg * 8);
+            if (my_i >= 0 && ks * 32 + lg * 8 < Dk)
+                raw = *reinterpret_cast<const uint4*>(qp + ks * 32 + lg * 8);
             qf[ks] = *reinterpret_cast<bf16x8_t*>(&raw);
         }
     }
@@ -645,35 +675,34 @@ window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __
     const int lo = max(0, i_min - window + 1);
     const int nfirst = min(keep, lo);
     const int n = nfirst + (i_max - lo + 1);
-    const long krow = (long)G * DK, vrow = (long)G * DV;
     float m_run = -INFINITY, l_run = 0.f;
-    f32x4_t o_acc[DV / 16];
+    f32x4_t o_acc[DVP / 16];
 #pragma unroll
-    for (int nb = 0; nb < DV / 16; ++nb) o_acc[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < DVP / 16; ++nb) o_acc[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     for (int base = 0; base < n; base += MA_KT) {
         // ---- stage K (row-major) and V (transposed) tiles
-        for (int c = tid; c < MA_KT * (DK / 8); c += 256) {
-            const int m = c / (DK / 8), part = c % (DK / 8);
+        for (int c = tid; c < MA_KT * (DKP / 8); c += 256) {
+            const int m = c / (DKP / 8), part = c % (DKP / 8);
             uint4 raw = make_uint4(0, 0, 0, 0);
-            if (base + m < n) {
+            if (base + m < n && part * 8 < Dk) {
                 const int mm = base + m;
                 const int j = mm < nfirst ? mm : lo + (mm - nfirst);
                 const int blk = bt[j / bsz];
                 const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
-                raw = *reinterpret_cast<const uint4*>(kc + slot * krow + (long)g * DK + part * 8);
+                raw = *reinterpret_cast<const uint4*>(kc + slot * ktok + (long)g * khead + part * 8);
             }
             *reinterpret_cast<uint4*>(k_lds + m * KS + part * 8) = raw;
         }
-        for (int c = tid; c < MA_KT * (DV / 8); c += 256) {
+        for (int c = tid; c < MA_KT * (DVP / 8); c += 256) {
             const int m = c % MA_KT, part = c / MA_KT;   // consecutive lanes: consecutive keys
             uint4 raw = make_uint4(0, 0, 0, 0);
-            if (base + m < n) {
+            if (base + m < n && part * 8 < Dv) {
                 const int mm = base + m;
                 const int j = mm < nfirst ? mm : lo + (mm - nfirst);
                 const int blk = bt[j / bsz];
                 const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
-                raw = *reinterpret_cast<const uint4*>(vc + slot * vrow + (long)g * DV + part * 8);
+                raw = *reinterpret_cast<const uint4*>(vc + slot * vtok + (long)g * vhead + part * 8);
             }
             const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -690,7 +719,7 @@ window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __
         for (int kb = 0; kb < 4; ++kb) {
             f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < DK / 32; ++ks) {
+            for (int ks = 0; ks < DKP / 32; ++ks) {
                 const bf16x8_t ka = *reinterpret_cast<const bf16x8_t*>(
                     k_lds + (kb * 16 + lr) * KS + ks * 32 + lg * 8);
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[ks], acc, 0, 0, 0);
@@ -702,7 +731,11 @@ window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __
                 const int dist = my_i - j;
                 const bool vis = mm < n && my_i >= 0 && dist >= 0 && (dist < window || j < keep);
                 float x = -INFINITY;
-                if (vis) x = acc[r] * scale - a1 * __logf(1.f + a2 * (float)dist);
+                if (vis) {
+                    x = acc[r] * qscale;
+                    if (r1) x -= a1 * __logf(1.f + a2 * (float)dist);
+                    if (cap > 0.f) x = cap * tanhf(x / cap);
+                }
                 sv[kb][r] = x;
                 mt = fmaxf(mt, x);
             }
@@ -736,7 +769,7 @@ window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __
 #pragma unroll
         for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, lg * 4 + r, WAVE);
 #pragma unroll
-        for (int nb = 0; nb < DV / 16; ++nb)
+        for (int nb = 0; nb < DVP / 16; ++nb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) o_acc[nb][r] *= cr[r];
         // ---- O += P V, 32 keys per product, P as hi + lo
@@ -751,7 +784,7 @@ window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __
                 pl.u[jj] = f2bf_rne(pv - __uint_as_float((uint32_t)hb << 16));
             }
 #pragma unroll
-            for (int nb = 0; nb < DV / 16; ++nb) {
+            for (int nb = 0; nb < DVP / 16; ++nb) {
                 union { bf16x8_t v; uint2 h[2]; } vb;
                 const uint16_t* vp = vt_lds + (nb * 16 + lr) * VS + 32 * kc2 + 4 * lg;
                 vb.h[0] = *reinterpret_cast<const uint2*>(vp);
@@ -762,20 +795,28 @@ window_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __
         }
         __syncthreads();
     }
-    // ---- epilogue: rows 4*lg + r of this wave, channel 16*nb + lr
+    // ---- epilogue: rows 4*lg + r of this wave, channel 16*nb + lr. A sink adds
+    // one term to the row's denominator (computed by the lane that owns the row)
+    float fin = l_run > 0.f ? 1.f / l_run : 0.f;
+    if (sink) {
+        const float sk = rsink[myrow];
+        const float mf = fmaxf(m_run, sk);
+        const float ca = m_run > -INFINITY ? expf(m_run - mf) : 0.f;
+        fin = ca / (l_run * ca + expf(sk - mf));
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int row = wv * 16 + lg * 4 + r;
-        const float lsum = __shfl(l_run, lg * 4 + r, WAVE);
+        const float inv = __shfl(fin, lg * 4 + r, WAVE);
         if (rpos[row] < 0) continue;
         const int tq = row / rep, h = g * rep + row % rep;
         const long tok = (long)b * S + t0 + tq;
-        const float inv = 1.f / lsum;
-        bf16* op = out + (tok * H + h) * (long)DV;
-        const bf16* gp = gate ? gate + tok * gstride + (long)h * DV : nullptr;
+        bf16* op = out + (tok * H + h) * (long)Dv;
+        const bf16* gp = gate ? gate + tok * gstride + (long)h * Dv : nullptr;
 #pragma unroll
-        for (int nb = 0; nb < DV / 16; ++nb) {
+        for (int nb = 0; nb < DVP / 16; ++nb) {
             const int d = nb * 16 + lr;
+            if (d >= Dv) continue;
             float o = o_acc[nb][r] * inv;
             if (gp) o *= sigmoidf_(__bfloat162float(gp[d]));
             op[d] = __float2bfloat16(o);
@@ -809,7 +850,7 @@ __global__ void delta_prep_kernel(const float* __restrict__ qkv, long cstride,
                                   const float* __restrict__ dt_bias,
                                   const float* __restrict__ a_log, const int* __restrict__ pos,
                                   const int* __restrict__ seq, float* __restrict__ prep, long PS,
-                                  long ntok, int S, int H, int G, int D) {
+                                  long ntok, int S, int H, int G, int D, int per_head) {
     const int lane = threadIdx.x & (WAVE - 1);
     const int units = 2 * G + H;
     const long wid = (long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
@@ -838,10 +879,16 @@ __global__ void delta_prep_kernel(const float* __restrict__ qkv, long cstride,
     } else {
         const int h = u - 2 * G;
         const float neg_rate = -expf(a_log[h]);
-        const T* ap = a + tok * astride + (long)h * D;
-        for (int i = lane; i < D; i += WAVE)
-            pr[(long)(2 * G + h) * D + i] =
-                expf(neg_rate * softplusf_(ldf<T>(ap + i) + dt_bias[h * D + i]));
+        if (per_head) {
+            // one decay for the whole head, broadcast over its key channels
+            const float dec = expf(neg_rate * softplusf_(ldf<T>(a + tok * astride + h) + dt_bias[h]));
+            for (int i = lane; i < D; i += WAVE) pr[(long)(2 * G + h) * D + i] = dec;
+        } else {
+            const T* ap = a + tok * astride + (long)h * D;
+            for (int i = lane; i < D; i += WAVE)
+                pr[(long)(2 * G + h) * D + i] =
+                    expf(neg_rate * softplusf_(ldf<T>(ap + i) + dt_bias[h * D + i]));
+        }
         if (lane == 0)
             pr[(long)(2 * G + H) * D + h] = sigmoidf_(ldf<T>(beta + tok * bstride + h));
     }
@@ -994,7 +1041,8 @@ template <typename T>
 __global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const T* __restrict__ gate,
                                      long gstride, const float* __restrict__ w, float eps,
                                      const int* __restrict__ pos, const int* __restrict__ seq,
-                                     T* __restrict__ out, long ntok, int S, int H, int Dv) {
+                                     T* __restrict__ out, long ntok, int S, int H, int Dv,
+                                     int gate_silu) {
     const int lane = threadIdx.x & (WAVE - 1);
     const long wid = (long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
     if (wid >= ntok * H) return;
@@ -1010,8 +1058,10 @@ __global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const T* __res
     for (int c = lane; c < Dv; c += WAVE) { float v = ip[c]; ss += v * v; }
     const float inv = 1.f / sqrtf(wave_sum(ss) / Dv + eps);
     const T* gp = gate + tok * gstride + (long)h * Dv;
-    for (int c = lane; c < Dv; c += WAVE)
-        stf<T>(op + c, ip[c] * inv * w[c] * sigmoidf_(ldf<T>(gp + c)));
+    for (int c = lane; c < Dv; c += WAVE) {
+        const float gv = ldf<T>(gp + c);
+        stf<T>(op + c, ip[c] * inv * w[c] * (gate_silu ? gv * sigmoidf_(gv) : sigmoidf_(gv)));
+    }
 }
 
 // ------------------------------------------------------------- elementwise
@@ -1064,6 +1114,128 @@ __global__ void gelu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ ou
         for (int e = 0; e < 8; ++e)
             o[e] = 0.5f * z[e] * (1.f + tanhf(0.7978845608028654f *
                                               (z[e] + 0.044715f * z[e] * z[e] * z[e]))) * u[e];
+        T* op = out + r * I + c;
+        if constexpr (sizeof(T) == 2) {
+            uint32_t pk[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                pk[e] = (uint32_t)f2bf_rne(o[2 * e]) | ((uint32_t)f2bf_rne(o[2 * e + 1]) << 16);
+            *reinterpret_cast<uint4*>(op) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        } else {
+            *reinterpret_cast<float4*>(op) = make_float4(o[0], o[1], o[2], o[3]);
+            *reinterpret_cast<float4*>(op + 4) = make_float4(o[4], o[5], o[6], o[7]);
+        }
+    }
+}
+
+
+// ------------------------------------------------------------------ RMS norm
+// x / sqrt(mean(x^2) + eps) * w (or * (1 + w)); one 256-thread workgroup per
+// row, fp32 statistics; input and output rows may be strided slices
+template <typename TIn, typename TOut>
+__global__ void __launch_bounds__(LN_THREADS)
+rms_norm_kernel(const TIn* __restrict__ x, long xs, const float* __restrict__ w, int one_plus,
+                float eps, TOut* __restrict__ out, long os, int C) {
+    __shared__ float red[LN_THREADS / WAVE];
+    const long row = blockIdx.x;
+    const TIn* xr = x + row * xs;
+    float s = 0.f;
+    for (int c = threadIdx.x; c < C; c += LN_THREADS) { const float v = ldf<TIn>(xr + c); s += v * v; }
+    const float inv = 1.f / sqrtf(block_sum(s, red) / C + eps);
+    TOut* o = out + row * os;
+    const float add = one_plus ? 1.f : 0.f;
+    for (int c = threadIdx.x; c < C; c += LN_THREADS)
+        stf<TOut>(o + c, ldf<TIn>(xr + c) * inv * (w[c] + add));
+}
+
+// post-norm residual step: stream[row] += rms_norm(y[row]) * (w | 1 + w), fp32;
+// optionally also writes the updated row in the next GEMM's input type
+template <typename TY, typename TC>
+__global__ void __launch_bounds__(LN_THREADS)
+add_rms_norm_kernel(float* __restrict__ stream, const TY* __restrict__ y,
+                    const float* __restrict__ w, int one_plus, float eps,
+                    TC* __restrict__ copy, int C) {
+    __shared__ float red[LN_THREADS / WAVE];
+    const long row = blockIdx.x;
+    const TY* yr = y + row * C;
+    float s = 0.f;
+    for (int c = threadIdx.x; c < C; c += LN_THREADS) { const float v = ldf<TY>(yr + c); s += v * v; }
+    const float inv = 1.f / sqrtf(block_sum(s, red) / C + eps);
+    const float add = one_plus ? 1.f : 0.f;
+    float* xr = stream + row * C;
+    for (int c = threadIdx.x; c < C; c += LN_THREADS) {
+        const float v = xr[c] + ldf<TY>(yr + c) * inv * (w[c] + add);
+        xr[c] = v;
+        if (copy) stf<TC>(copy + row * C + c, v);
+    }
+}
+
+// ---------------------------------------------------------- rotary positions
+// pairs (2i, 2i+1) of the first 2*half channels of every head turn by
+// p * inv_freq[i] (fp32 angle, full-range sincosf); the rest is copied.
+// One thread per (token, head, channel pair or trailing channel).
+template <typename TIn, typename TOut>
+__global__ void rope_pairs_kernel(const TIn* __restrict__ x, long xt, long xh,
+                                  TOut* __restrict__ out, long ot, long oh,
+                                  const int* __restrict__ pos, const float* __restrict__ inv_freq,
+                                  int half, long ntok, int N, int C) {
+    const int per = half + (C - 2 * half);            // work items per head
+    const long total = ntok * N * per;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int e = idx % per;
+        const long th = idx / per;
+        const int h = th % N;
+        const long tok = th / N;
+        const int p = pos[tok];
+        const TIn* xp = x + tok * xt + (long)h * xh;
+        TOut* op = out + tok * ot + (long)h * oh;
+        if (e < half) {
+            float a = ldf<TIn>(xp + 2 * e), b = ldf<TIn>(xp + 2 * e + 1);
+            float sn, cs;
+            sincosf((float)(p < 0 ? 0 : p) * inv_freq[e], &sn, &cs);
+            stf<TOut>(op + 2 * e, a * cs - b * sn);
+            stf<TOut>(op + 2 * e + 1, b * cs + a * sn);
+        } else {
+            const int c = 2 * half + (e - half);
+            stf<TOut>(op + c, ldf<TIn>(xp + c));
+        }
+    }
+}
+
+// ------------------------------------------------------- clamped gated unit
+// out[r, c] = g * sigmoid(alpha * g) * (u + 1), g = min(gu[r, c], limit),
+// u = clamp(gu[r, I + c], -limit, limit)
+DEV float clamped_glu_(float g, float u, float limit, float alpha) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * sigmoidf_(alpha * g) * (u + 1.f);
+}
+
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, long rows, int I,
+                                   float limit, float alpha) {
+    const long total = rows * I;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / I;
+        const int c = idx % I;
+        stf<T>(out + idx, clamped_glu_(ldf<T>(gu + r * 2 * I + c), ldf<T>(gu + r * 2 * I + I + c),
+                                       limit, alpha));
+    }
+}
+
+template <typename T>
+__global__ void clamped_glu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, long rows,
+                                       int I, float limit, float alpha) {
+    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (c >= I) return;
+    for (long r = blockIdx.y; r < rows; r += gridDim.y) {
+        float z[8], u[8], o[8];
+        load8<T>(gu + r * 2 * I + c, z);
+        load8<T>(gu + r * 2 * I + I + c, u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = clamped_glu_(z[e], u[e], limit, alpha);
         T* op = out + r * I + c;
         if constexpr (sizeof(T) == 2) {
             uint32_t pk[4];
@@ -1162,31 +1334,46 @@ int nx_paged_kv_write(void* kc, void* vc, const void* k, long kstride, const voi
     return (int)hipGetLastError();
 }
 
-int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, const int* pos,
-                   const int* seq, const int* btab, int max_blocks, const float* r1,
-                   const float* r2, const void* gate, long gstride, void* out, int io_bf16,
-                   int out_bf16, int B, int S, int H, int G, int Dk, int Dv, int bsz,
-                   float scale, int window, int keep, hipStream_t st) {
+int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long khead,
+                  const void* vc, long vtok, long vhead, const int* pos, const int* seq,
+                  const int* btab, int max_blocks, const float* r1, const float* r2,
+                  const float* sink, const void* gate, long gstride, void* out, int io_bf16,
+                  int out_bf16, int B, int S, int H, int G, int Dk, int Dv, int bsz,
+                  float scale, int window, int keep, float cap, float qt_coef, int qt_every,
+                  hipStream_t st) {
     if ((long)B * S <= 0) return 0;
-    if (Dv > WAVE * 4 || H % G != 0) return -1;
+    if (Dv > WAVE * 8 || H % G != 0 || Dk <= 0 || Dv <= 0) return -1;
     if (!io_bf16 && out_bf16) return -2;
+    if ((r1 == nullptr) != (r2 == nullptr)) return -4;
+    const int esz = io_bf16 ? 2 : 4;
+    const int vecn = 16 / esz;                            // elements per 16-byte load
+    const bool k_al = (Dk % 8) == 0 && (ktok % vecn) == 0 && (khead % vecn) == 0 &&
+                      ((uintptr_t)kc % 16) == 0;
+    const bool v_al = (Dv % 8) == 0 && (vtok % vecn) == 0 && (vhead % vecn) == 0 &&
+                      ((uintptr_t)vc % 16) == 0;
     {
-        // matrix-core path: bf16 steps with prompt portions, common head shapes
+        // matrix-core path: bf16 steps with prompt portions, head sizes up to
+        // 192 (keys) / 128 (values) in multiples of 8
         const int rp = H / G;
         const bool rep_ok = rp <= MA_ROWS;       // rows beyond QT*rep stay idle
-        const bool dk_ok = Dk == 32 || Dk == 64 || Dk == 128;
-        const bool dv_ok = Dv == 32 || Dv == 64 || Dv == 128;
-        if (io_bf16 && out_bf16 && S > 1 && rep_ok && dk_ok && dv_ok && (qstride % 8) == 0 &&
-            ((uintptr_t)q % 16) == 0) {
+        const int dkp = (Dk + 31) & ~31, dvp = (Dv + 31) & ~31;
+        const bool dk_ok = dkp <= 128 || dkp == 192;
+        const bool dv_ok = dvp <= 128;
+        if (io_bf16 && out_bf16 && S > 1 && rep_ok && dk_ok && dv_ok && k_al && v_al &&
+            (qstride % 8) == 0 && ((uintptr_t)q % 16) == 0) {
             const int QTm = MA_ROWS / rp;
             dim3 gm((S + QTm - 1) / QTm, G, B), bm(256);
-#define MA(DKV, DVV) window_attn_mfma_kernel<DKV, DVV><<<gm, bm, 0, st>>>( \
+#define MA(DKV, DVV) paged_attn_mfma_kernel<DKV, DVV><<<gm, bm, 0, st>>>( \
         (const bf16*)q, qstride, (const bf16*)kc, (const bf16*)vc, pos, seq, btab, max_blocks, \
-        r1, r2, (const bf16*)gate, gstride, (bf16*)out, H, G, bsz, S, scale, window, keep, QTm)
-#define MAV(DKV) do { if (Dv == 32) MA(DKV, 32); else if (Dv == 64) MA(DKV, 64); else MA(DKV, 128); } while (0)
-            if (Dk == 32) MAV(32);
-            else if (Dk == 64) MAV(64);
-            else MAV(128);
+        r1, r2, (const bf16*)gate, gstride, (bf16*)out, H, G, Dk, Dv, bsz, S, scale, window, \
+        keep, QTm, ktok, khead, vtok, vhead, sink, cap, qt_coef, qt_every)
+#define MAV(DKV) do { if (dvp == 32) MA(DKV, 32); else if (dvp == 64) MA(DKV, 64); \
+                      else if (dvp == 96) MA(DKV, 96); else MA(DKV, 128); } while (0)
+            if (dkp == 32) MAV(32);
+            else if (dkp == 64) MAV(64);
+            else if (dkp == 96) MAV(96);
+            else if (dkp == 128) MAV(128);
+            else MAV(192);
 #undef MAV
 #undef MA
             return (int)hipGetLastError();
@@ -1202,7 +1389,7 @@ int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, 
     dim3 grid((S + QT - 1) / QT, G * chunks, B), block(NW * WAVE);
     // decode shape: 8 value channels per lane when they tile a wave evenly
     int lpr = 0;
-    if (dec && (Dv % 8) == 0) {
+    if (dec && v_al) {
         const int l = Dv / 8;
         if (l <= WAVE && (l & (l - 1)) == 0) lpr = l;
     }
@@ -1217,12 +1404,14 @@ int nx_window_attn(const void* q, long qstride, const void* kc, const void* vc, 
         sh = (size_t)(NQ * DkP + (ptile > marea ? ptile : marea)) * sizeof(float);
     }
     if (sh > 60 * 1024) return -3;
+    const int kvec = k_al ? 1 : 0;
 #define WA(T, TO, MR, Q, W) window_attn_kernel<T, TO, MR, Q, W><<<grid, block, sh, st>>>( \
         (const T*)q, qstride, (const T*)kc, (const T*)vc, pos, seq, btab, max_blocks, r1, r2, \
         (const T*)gate, gstride, (TO*)out, H, G, Dk, Dv, bsz, S, scale, window, keep, HPW, QT, \
-        chunks, lpr, pws)
+        chunks, lpr, pws, ktok, khead, vtok, vhead, kvec, sink, cap, qt_coef, qt_every)
 #define WAS(T, TO, MR) do { if (dec) WA(T, TO, MR, 4, 16); else WA(T, TO, MR, 16, 4); } while (0)
-#define WAM(T, TO) do { if (Dv <= 2 * WAVE) WAS(T, TO, 2); else WAS(T, TO, 4); } while (0)
+#define WAM(T, TO) do { if (Dv <= 2 * WAVE) WAS(T, TO, 2); else if (Dv <= 4 * WAVE) WAS(T, TO, 4); \
+                        else WAS(T, TO, 8); } while (0)
     if (io_bf16 && out_bf16) WAM(bf16, bf16);
     else if (io_bf16) WAM(bf16, float);
     else WAM(float, float);
@@ -1237,7 +1426,7 @@ int nx_gated_delta(const float* qkv, long cstride, const void* beta, long bstrid
                    const float* a_log, const float* norm_w, float eps, float* state,
                    const int* pos, const int* seq, const int* nvalid, float* prep, long PS,
                    float* obuf, void* out, int in_bf16, int B, int S, int H, int G, int D,
-                   int Dv, hipStream_t st) {
+                   int Dv, int per_head, int gate_silu, hipStream_t st) {
     if (B <= 0 || S <= 0) return 0;
     if (D > 256 || H % G != 0 || PS < (long)(2 * G + H) * D + H + G) return -1;
     const long ntok = (long)B * S;
@@ -1246,10 +1435,10 @@ int nx_gated_delta(const float* qkv, long cstride, const void* beta, long bstrid
         dim3 g0((unsigned)((waves + 3) / 4)), b0(4 * WAVE);
         if (in_bf16) delta_prep_kernel<bf16><<<g0, b0, 0, st>>>(
             qkv, cstride, (const bf16*)beta, bstride, (const bf16*)a, astride, dt_bias, a_log,
-            pos, seq, prep, PS, ntok, S, H, G, D);
+            pos, seq, prep, PS, ntok, S, H, G, D, per_head);
         else delta_prep_kernel<float><<<g0, b0, 0, st>>>(
             qkv, cstride, (const float*)beta, bstride, (const float*)a, astride, dt_bias, a_log,
-            pos, seq, prep, PS, ntok, S, H, G, D);
+            pos, seq, prep, PS, ntok, S, H, G, D, per_head);
         int rc = (int)hipGetLastError();
         if (rc) return rc;
     }
@@ -1268,9 +1457,11 @@ int nx_gated_delta(const float* qkv, long cstride, const void* beta, long bstrid
     const long waves = ntok * H;
     dim3 g2((unsigned)((waves + 3) / 4)), b2(4 * WAVE);
     if (in_bf16) gated_rmsnorm_kernel<bf16><<<g2, b2, 0, st>>>(
-        obuf, (const bf16*)gate, gstride, norm_w, eps, pos, seq, (bf16*)out, ntok, S, H, Dv);
+        obuf, (const bf16*)gate, gstride, norm_w, eps, pos, seq, (bf16*)out, ntok, S, H, Dv,
+        gate_silu);
     else gated_rmsnorm_kernel<float><<<g2, b2, 0, st>>>(
-        obuf, (const float*)gate, gstride, norm_w, eps, pos, seq, (float*)out, ntok, S, H, Dv);
+        obuf, (const float*)gate, gstride, norm_w, eps, pos, seq, (float*)out, ntok, S, H, Dv,
+        gate_silu);
     return (int)hipGetLastError();
 }
 
@@ -1304,6 +1495,67 @@ int nx_gelu_mul(const void* gu, void* out, int is_bf16, long rows, int I, hipStr
     dim3 grid(grid_for(rows * I, 256)), block(256);
     if (is_bf16) gelu_mul_kernel<bf16><<<grid, block, 0, st>>>((const bf16*)gu, (bf16*)out, rows, I);
     else gelu_mul_kernel<float><<<grid, block, 0, st>>>((const float*)gu, (float*)out, rows, I);
+    return (int)hipGetLastError();
+}
+
+int nx_rms_norm(const void* x, long xs, int x_bf16, const float* w, int one_plus, float eps,
+                void* out, long os, int out_bf16, long rows, int C, hipStream_t st) {
+    if (rows <= 0) return 0;
+    dim3 grid((unsigned)rows), block(LN_THREADS);
+#define RN(TI, TO) rms_norm_kernel<TI, TO><<<grid, block, 0, st>>>( \
+        (const TI*)x, xs, w, one_plus, eps, (TO*)out, os, C)
+    if (x_bf16 && out_bf16) RN(bf16, bf16);
+    else if (x_bf16) RN(bf16, float);
+    else if (out_bf16) RN(float, bf16);
+    else RN(float, float);
+#undef RN
+    return (int)hipGetLastError();
+}
+
+int nx_add_rms_norm(float* stream, const void* y, int y_bf16, const float* w, int one_plus,
+                    float eps, void* copy_bf16, long rows, int C, hipStream_t st) {
+    if (rows <= 0) return 0;
+    dim3 grid((unsigned)rows), block(LN_THREADS);
+    if (y_bf16) add_rms_norm_kernel<bf16, bf16><<<grid, block, 0, st>>>(
+        stream, (const bf16*)y, w, one_plus, eps, (bf16*)copy_bf16, C);
+    else add_rms_norm_kernel<float, bf16><<<grid, block, 0, st>>>(
+        stream, (const float*)y, w, one_plus, eps, (bf16*)copy_bf16, C);
+    return (int)hipGetLastError();
+}
+
+int nx_rope_pairs(const void* x, long xt, long xh, int x_bf16, void* out, long ot, long oh,
+                  int out_bf16, const int* pos, const float* inv_freq, int half, long ntok,
+                  int N, int C, hipStream_t st) {
+    const long total = ntok * N * (C - half);
+    if (total <= 0) return 0;
+    if (2 * half > C) return -1;
+    dim3 grid(grid_for(total, 256)), block(256);
+#define RP(TI, TO) rope_pairs_kernel<TI, TO><<<grid, block, 0, st>>>( \
+        (const TI*)x, xt, xh, (TO*)out, ot, oh, pos, inv_freq, half, ntok, N, C)
+    if (x_bf16 && out_bf16) RP(bf16, bf16);
+    else if (x_bf16) RP(bf16, float);
+    else if (out_bf16) RP(float, bf16);
+    else RP(float, float);
+#undef RP
+    return (int)hipGetLastError();
+}
+
+int nx_clamped_glu(const void* gu, void* out, int is_bf16, long rows, int I, float limit,
+                   float alpha, hipStream_t st) {
+    if (rows <= 0) return 0;
+    if ((I % 8) == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+        dim3 gv((I / 8 + 255) / 256, (unsigned)(rows > 32768 ? 32768 : rows)), bv(256);
+        if (is_bf16) clamped_glu_vec_kernel<bf16><<<gv, bv, 0, st>>>(
+            (const bf16*)gu, (bf16*)out, rows, I, limit, alpha);
+        else clamped_glu_vec_kernel<float><<<gv, bv, 0, st>>>(
+            (const float*)gu, (float*)out, rows, I, limit, alpha);
+        return (int)hipGetLastError();
+    }
+    dim3 grid(grid_for(rows * I, 256)), block(256);
+    if (is_bf16) clamped_glu_kernel<bf16><<<grid, block, 0, st>>>(
+        (const bf16*)gu, (bf16*)out, rows, I, limit, alpha);
+    else clamped_glu_kernel<float><<<grid, block, 0, st>>>(
+        (const float*)gu, (float*)out, rows, I, limit, alpha);
     return (int)hipGetLastError();
 }
 
