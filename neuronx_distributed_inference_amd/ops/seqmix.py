@@ -132,9 +132,18 @@ def _rows_view(t: torch.Tensor):
     (a column slice of a fused GEMM output qualifies): returns row stride."""
     assert t.stride(-1) == 1, "innermost dim must be contiguous"
     if t.dim() == 3:
-        assert t.stride(0) == t.stride(1) * t.shape[1], "rows must be uniformly strided"
-        return t.stride(1)
+        return _token_stride(t)
     return t.stride(0)
+
+
+def _token_stride(t: torch.Tensor) -> int:
+    """Stride between consecutive tokens of a (B, S, ...) tensor whose
+    tokens are uniformly strided (a size-1 axis has no stride of its own)."""
+    B, S = t.shape[0], t.shape[1]
+    if S == 1:
+        return t.stride(0) if B > 1 else max(t.stride(0), t.stride(1))
+    assert B == 1 or t.stride(0) == t.stride(1) * S, "rows must be uniformly strided"
+    return t.stride(1)
 
 
 class StepLayout:
@@ -429,12 +438,12 @@ def rotate_interleaved(x, step: StepLayout, inv_freq, out=None, out_dtype=None):
         B, S, N, C = x.shape
         if out is None:
             out = torch.empty(B, S, N, C, dtype=out_dtype, device=x.device)
-        for t in (x, out):
-            assert t.stride(3) == 1 and t.stride(0) == t.stride(1) * S
+        assert x.stride(3) == 1 and out.stride(3) == 1
         assert 2 * inv_freq.numel() <= C
         _check(lib.nx_rope_pairs(
-            _p(x), ctypes.c_long(x.stride(1)), ctypes.c_long(x.stride(2)), _is_bf16(x),
-            _p(out), ctypes.c_long(out.stride(1)), ctypes.c_long(out.stride(2)), _is_bf16(out),
+            _p(x), ctypes.c_long(_token_stride(x)), ctypes.c_long(x.stride(2)), _is_bf16(x),
+            _p(out), ctypes.c_long(_token_stride(out)), ctypes.c_long(out.stride(2)),
+            _is_bf16(out),
             _p(step.positions), _p(_f32(inv_freq)), inv_freq.numel(),
             ctypes.c_long(B * S), N, C, _stream()), "rotate_interleaved")
         return out

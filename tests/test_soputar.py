@@ -541,8 +541,12 @@ def test_prefill_decode_portions_match_oracle(device, make):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-def test_residual_stream_per_layer(device):
-    cfg = varied_cfg()
+@pytest.mark.parametrize("make,tol", [(model_cfg, 3e-5), (varied_cfg, 1e-3)])
+def test_residual_stream_per_layer(device, make, tol):
+    """The stream after every layer. (The second configuration normalises
+    read-outs that nearly cancel in its first tokens, which magnifies fp32
+    rounding; its bound is looser for that reason only.)"""
+    cfg = make()
     W = make_weights(cfg, seed=7)
     toks = tokens_for(cfg, 9, seed=8)
     _, streams = oracle.forward(cfg, W, toks, return_layers=True)
@@ -556,7 +560,7 @@ def test_residual_stream_per_layer(device):
         hk.remove()
     assert len(seen) == streams.shape[0] == len(cfg["layers"])
     for r, s in enumerate(seen):
-        close(s[0], streams[r], 3e-4, rtol=1e-4)
+        close(s[0], streams[r], tol)
 
 
 @pytest.mark.parametrize("device", DEVICES)
