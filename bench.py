@@ -69,8 +69,11 @@ def parse_args():
                    help="fused speculative decoding: --model target + 1b draft, spec-len 5")
     p.add_argument("--spec-len", type=int, default=5)
     p.add_argument("--hybrid", action="store_true",
-                   help="Nabelix (windowed attention + gated delta rule) prefill/decode "
-                        "throughput beside Llama at equal width/depth/ff/vocab")
+                   help="prefill/decode throughput of the hybrid decoders (Nabelix: windowed "
+                        "attention + gated delta rule; Soputar: latent, delta-rule and capped "
+                        "attention layers) beside Llama at equal width/depth/ff/vocab")
+    p.add_argument("--hybrid-models", default="llama,nabelix,soputar",
+                   help="comma-separated subset of llama,nabelix,soputar for --hybrid")
     p.add_argument("--hybrid-sizes", default="2048,4096",
                    help="comma-separated layer widths for --hybrid")
     p.add_argument("--hybrid-layers", type=int, default=4)
@@ -104,6 +107,9 @@ def run_hybrid_bench(args):
     from neuronx_distributed_inference_amd.models.nabelix.modeling_nabelix import (
         NabelixForCausalLM, NabelixInferenceConfig,
     )
+    from neuronx_distributed_inference_amd.models.soputar.modeling_soputar import (
+        SoputarForCausalLM, SoputarInferenceConfig,
+    )
 
     dtype = "bfloat16" if on_gpu else "float32"
     B, ctx, steps, warmup = args.batch_per_gpu, args.ctx, args.steps, args.warmup
@@ -132,6 +138,33 @@ def run_hybrid_bench(args):
                 rms_norm_eps=1e-5, rope_theta=500000.0, hidden_act="silu",
                 tie_word_embeddings=False)
             cls = LlamaForCausalLM
+        elif kind == "soputar":
+            # the design's layer mix, repeated to depth L: latent attention
+            # (512-wide latent + 64 rotated channels), delta rule, capped
+            # GQA attention, and a layer that borrows the previous one's KV
+            mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+            att = {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                   "softcap": 20.0, "q_temp": {"coef": 0.5, "every": 64}}
+            quad = [
+                {"type": "latent_attention", "mlp": mlp, "mixer": {
+                    "heads": H, "dim": 128, "rot_dim": 64, "vdim": 128,
+                    "kv_rank": min(512, width // 4),
+                    "scale": 192 ** -0.5, "rot": {"base": 10000.0, "dims": 64}}},
+                {"type": "delta", "mlp": mlp, "mixer": {
+                    "heads": H, "kv_heads": H, "dim": 128, "vdim": 128, "conv": 4}},
+                {"type": "attention", "mlp": mlp, "mixer": dict(att)},
+                {"type": "attention", "mlp": mlp, "mixer": dict(att, kv_from=2)},
+            ]
+            layers = []
+            for i in range(L):
+                lc = json.loads(json.dumps(quad[i % 4]))
+                if "kv_from" in lc["mixer"]:
+                    lc["mixer"]["kv_from"] = i - 1
+                layers.append(lc)
+            cfg = SoputarInferenceConfig(
+                neuron_config=ec, architecture="Soputar", width=width, vocab=V,
+                layers=layers, norm={"eps": 1e-5}, embedding={"scale": width ** 0.5})
+            cls = SoputarForCausalLM
         else:
             layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff}, "mixer": {
                 "left": {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128,
@@ -159,7 +192,8 @@ def run_hybrid_bench(args):
         return m
 
     for width in [int(x) for x in args.hybrid_sizes.split(",")]:
-        for kind in ("llama", "nabelix"):
+        for kind in [k for k in ("llama", "nabelix", "soputar")
+                     if k in args.hybrid_models.split(",")]:
             with torch.inference_mode():
                 # ---- prefill: one prompt, three timed repetitions
                 m = build(kind, width, 1)

@@ -162,6 +162,15 @@ class RecurrentStateManager(nn.Module):
     def estimate_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.tensors.values())
 
+    def snapshot(self):
+        """Copies of every state tensor (for steps that must be undone, e.g.
+        the warm-up runs of a graph capture on live inputs)."""
+        return {k: t.data.clone() for k, t in self.tensors.items()}
+
+    def restore(self, snap):
+        for k, v in snap.items():
+            self.tensors[k].data.copy_(v)
+
     def reset(self):
         for t in self.tensors.values():
             t.data.zero_()

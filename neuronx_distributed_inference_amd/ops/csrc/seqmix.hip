@@ -605,11 +605,14 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
 // temperature, bias, cap, mask and online softmax are fp32 per lane; P enters the
 // second product as a hi + lo bf16 pair (16 mantissa bits), V as stored.
 // DKP / DVP are the head sizes padded to multiples of 32; the true Dk, Dv (any
-// multiples of 8) come at run time and the padding is zero-filled in LDS.
+// multiples of 8) come at run time and the padding is zero-filled in LDS. KT is
+// the key tile (64, or 32 for wide keys so that the K tile still fits LDS). Values
+// wider than DVP are split over `nsplit` workgroups that each recompute the scores
+// and own DVP value channels (latent caches: a 576-wide key row whose first 512
+// channels are the value).
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 #define MA_ROWS 64
-#define MA_KT 64
 
 DEV uint16_t f2bf_rne(float f) {
     uint32_t u = __float_as_uint(f);
@@ -617,7 +620,7 @@ DEV uint16_t f2bf_rne(float f) {
     return (uint16_t)(u >> 16);
 }
 
-template <int DKP, int DVP>
+template <int DKP, int DVP, int MA_KT>
 __global__ void __launch_bounds__(256)
 paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __restrict__ kc,
                        const bf16* __restrict__ vc, const int* __restrict__ pos,
@@ -627,7 +630,8 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
                        long gstride, bf16* __restrict__ out, int H, int G, int Dk, int Dv,
                        int bsz, int S, float scale, int window, int keep, int QT, long ktok,
                        long khead, long vtok, long vhead, const float* __restrict__ sink,
-                       float cap, float qt_coef, int qt_every) {
+                       float cap, float qt_coef, int qt_every, int nsplit) {
+    constexpr int KB = MA_KT / 16;           // 16-key score blocks per tile
     constexpr int KS = DKP + 8;              // K tile row stride (elements)
     constexpr int VS = MA_KT + 8;            // V^T tile row stride
     __shared__ __attribute__((aligned(16))) uint16_t k_lds[MA_KT * KS];
@@ -636,7 +640,9 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
     __shared__ float ra1[MA_ROWS], ra2[MA_ROWS], rsink[MA_ROWS];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int lr = lane & 15, lg = lane >> 4;
-    const int b = blockIdx.z, g = blockIdx.y, t0 = blockIdx.x * QT;
+    const int b = blockIdx.z, g = blockIdx.y / nsplit, t0 = blockIdx.x * QT;
+    const int dv0 = (blockIdx.y % nsplit) * DVP;         // first value channel of this split
+    const int dvn = min(DVP, Dv - dv0);
     const int rep = H / G;
     if (seq[b] < 0) return;
     if (tid < MA_ROWS) {
@@ -697,12 +703,13 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         for (int c = tid; c < MA_KT * (DVP / 8); c += 256) {
             const int m = c % MA_KT, part = c / MA_KT;   // consecutive lanes: consecutive keys
             uint4 raw = make_uint4(0, 0, 0, 0);
-            if (base + m < n && part * 8 < Dv) {
+            if (base + m < n && part * 8 < dvn) {
                 const int mm = base + m;
                 const int j = mm < nfirst ? mm : lo + (mm - nfirst);
                 const int blk = bt[j / bsz];
                 const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
-                raw = *reinterpret_cast<const uint4*>(vc + slot * vtok + (long)g * vhead + part * 8);
+                raw = *reinterpret_cast<const uint4*>(vc + slot * vtok + (long)g * vhead + dv0 +
+                                                      part * 8);
             }
             const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -713,10 +720,10 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         }
         __syncthreads();
         // ---- S^T = K Q^T: lane gets keys 16*kb + 4*lg + r of its own row lr
-        float sv[4][4];
+        float sv[KB][4];
         float mt = -INFINITY;
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb) {
+        for (int kb = 0; kb < KB; ++kb) {
             f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < DKP / 32; ++ks) {
@@ -747,7 +754,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         if (m_new > -INFINITY) {
             corr = expf(m_run - m_new);
 #pragma unroll
-            for (int kb = 0; kb < 4; ++kb)
+            for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const float pv = sv[kb][r] > -INFINITY ? expf(sv[kb][r] - m_new) : 0.f;
@@ -756,7 +763,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
                 }
         } else {
 #pragma unroll
-            for (int kb = 0; kb < 4; ++kb)
+            for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) sv[kb][r] = 0.f;
         }
@@ -774,7 +781,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
             for (int r = 0; r < 4; ++r) o_acc[nb][r] *= cr[r];
         // ---- O += P V, 32 keys per product, P as hi + lo
 #pragma unroll
-        for (int kc2 = 0; kc2 < 2; ++kc2) {
+        for (int kc2 = 0; kc2 < MA_KT / 32; ++kc2) {
             union { bf16x8_t v; uint16_t u[8]; } ph, pl;
 #pragma unroll
             for (int jj = 0; jj < 8; ++jj) {
@@ -811,12 +818,12 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         if (rpos[row] < 0) continue;
         const int tq = row / rep, h = g * rep + row % rep;
         const long tok = (long)b * S + t0 + tq;
-        bf16* op = out + (tok * H + h) * (long)Dv;
-        const bf16* gp = gate ? gate + tok * gstride + (long)h * Dv : nullptr;
+        bf16* op = out + (tok * H + h) * (long)Dv + dv0;
+        const bf16* gp = gate ? gate + tok * gstride + (long)h * Dv + dv0 : nullptr;
 #pragma unroll
         for (int nb = 0; nb < DVP / 16; ++nb) {
             const int d = nb * 16 + lr;
-            if (d >= Dv) continue;
+            if (d >= dvn) continue;
             float o = o_acc[nb][r] * inv;
             if (gp) o *= sigmoidf_(__bfloat162float(gp[d]));
             op[d] = __float2bfloat16(o);
@@ -1352,24 +1359,36 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
     const bool v_al = (Dv % 8) == 0 && (vtok % vecn) == 0 && (vhead % vecn) == 0 &&
                       ((uintptr_t)vc % 16) == 0;
     {
-        // matrix-core path: bf16 steps with prompt portions, head sizes up to
-        // 192 (keys) / 128 (values) in multiples of 8
+        // matrix-core path: bf16 steps with prompt portions (any head sizes in
+        // multiples of 8: keys up to 640 wide, wide values split over
+        // workgroups), and single-token steps of wide multi-query layers, whose
+        // many heads per cache row fill the 16-row tiles
         const int rp = H / G;
         const bool rep_ok = rp <= MA_ROWS;       // rows beyond QT*rep stay idle
         const int dkp = (Dk + 31) & ~31, dvp = (Dv + 31) & ~31;
-        const bool dk_ok = dkp <= 128 || dkp == 192;
-        const bool dv_ok = dvp <= 128;
-        if (io_bf16 && out_bf16 && S > 1 && rep_ok && dk_ok && dv_ok && k_al && v_al &&
+        const bool wide = dkp > 192 || dvp > 128;
+        const bool dk_ok = dkp <= 640;
+        const bool steps_ok = S > 1 || (wide && rp >= 8);
+        if (io_bf16 && out_bf16 && steps_ok && rep_ok && dk_ok && k_al && v_al &&
             (qstride % 8) == 0 && ((uintptr_t)q % 16) == 0) {
             const int QTm = MA_ROWS / rp;
-            dim3 gm((S + QTm - 1) / QTm, G, B), bm(256);
-#define MA(DKV, DVV) paged_attn_mfma_kernel<DKV, DVV><<<gm, bm, 0, st>>>( \
+            const int nsplit = wide ? (Dv + 127) / 128 : 1;
+            dim3 gm((S + QTm - 1) / QTm, G * nsplit, B), bm(256);
+#define MA(DKV, DVV, KTV) paged_attn_mfma_kernel<DKV, DVV, KTV><<<gm, bm, 0, st>>>( \
         (const bf16*)q, qstride, (const bf16*)kc, (const bf16*)vc, pos, seq, btab, max_blocks, \
         r1, r2, (const bf16*)gate, gstride, (bf16*)out, H, G, Dk, Dv, bsz, S, scale, window, \
-        keep, QTm, ktok, khead, vtok, vhead, sink, cap, qt_coef, qt_every)
-#define MAV(DKV) do { if (dvp == 32) MA(DKV, 32); else if (dvp == 64) MA(DKV, 64); \
-                      else if (dvp == 96) MA(DKV, 96); else MA(DKV, 128); } while (0)
-            if (dkp == 32) MAV(32);
+        keep, QTm, ktok, khead, vtok, vhead, sink, cap, qt_coef, qt_every, nsplit)
+#define MAV(DKV) do { if (dvp == 32) MA(DKV, 32, 64); else if (dvp == 64) MA(DKV, 64, 64); \
+                      else if (dvp == 96) MA(DKV, 96, 64); else MA(DKV, 128, 64); } while (0)
+            if (wide) {
+                if (dkp <= 128) MA(128, 128, 64);
+                else if (dkp <= 192) MA(192, 128, 64);
+                else if (dkp <= 256) MA(256, 128, 32);
+                else if (dkp <= 384) MA(384, 128, 32);
+                else if (dkp <= 576) MA(576, 128, 32);
+                else MA(640, 128, 32);
+            }
+            else if (dkp == 32) MAV(32);
             else if (dkp == 64) MAV(64);
             else if (dkp == 96) MAV(96);
             else if (dkp == 128) MAV(128);
@@ -1403,13 +1422,17 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
         ptile = (long)NW * pws;
         sh = (size_t)(NQ * DkP + (ptile > marea ? ptile : marea)) * sizeof(float);
     }
-    if (sh > 60 * 1024) return -3;
+    if (sh > 150 * 1024) return -3;
     const int kvec = k_al ? 1 : 0;
-#define WA(T, TO, MR, Q, W) window_attn_kernel<T, TO, MR, Q, W><<<grid, block, sh, st>>>( \
+    // beyond the default 64 KB of dynamic LDS a kernel has to be told its limit
+#define WA(T, TO, MR, Q, W) if (sh > 60 * 1024 && hipFuncSetAttribute( \
+        (const void*)window_attn_kernel<T, TO, MR, Q, W>, \
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh) != hipSuccess) return -5; \
+    window_attn_kernel<T, TO, MR, Q, W><<<grid, block, sh, st>>>( \
         (const T*)q, qstride, (const T*)kc, (const T*)vc, pos, seq, btab, max_blocks, r1, r2, \
         (const T*)gate, gstride, (TO*)out, H, G, Dk, Dv, bsz, S, scale, window, keep, HPW, QT, \
         chunks, lpr, pws, ktok, khead, vtok, vhead, kvec, sink, cap, qt_coef, qt_every)
-#define WAS(T, TO, MR) do { if (dec) WA(T, TO, MR, 4, 16); else WA(T, TO, MR, 16, 4); } while (0)
+#define WAS(T, TO, MR) do { if (dec) { WA(T, TO, MR, 4, 16); } else { WA(T, TO, MR, 16, 4); } } while (0)
 #define WAM(T, TO) do { if (Dv <= 2 * WAVE) WAS(T, TO, 2); else if (Dv <= 4 * WAVE) WAS(T, TO, 4); \
                         else WAS(T, TO, 8); } while (0)
     if (io_bf16 && out_bf16) WAM(bf16, bf16);

@@ -361,7 +361,15 @@ class ServingEngine:
                                phase="token_generation", block_table=bt)
                     return t if t is not None else lg
                 ex = (ids, pos, seq_ids, sp, block_table)
+            # capture warms the step up on the live inputs first. Rewriting
+            # a KV row with the same token is harmless, advancing a
+            # recurrence by it again is not: hold the recurrent state aside
+            # and put it back before the first replay
+            state = getattr(self.kv_mgr, "state", None)
+            saved = state.snapshot() if state is not None else None
             self._decode_graph = GraphRunner(fn, ex)
+            if saved is not None:
+                state.restore(saved)
             self._decode_graph_has_sp = sp is not None
         args = (ids, pos, seq_ids) + ((sp,) if self._decode_graph_has_sp else ()) \
             + (block_table,)

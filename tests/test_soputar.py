@@ -463,6 +463,10 @@ def test_latent_attention_far_keys_and_positions(device, cuts):
     (latent_cfg(4, 32, 16, 32, 64, scale=0.1), None),
     (latent_cfg(4, 32, 16, 80, 64, scale=0.1), [3, 60, 1, 66]),      # 80-wide rows
     (latent_cfg(2, 64, 32, 64, 96, scale=0.08, dims=16), [64, 66]),
+    # wide rows: 32-key tiles, values split over workgroups, also when decoding
+    (latent_cfg(8, 32, 32, 48, 224, scale=0.1), [70, 50] + [1] * 10),
+    (latent_cfg(16, 64, 64, 64, 512, scale=0.07), [100] + [1] * 30),
+    (latent_cfg(4, 16, 8, 16, 200, scale=0.1), [129, 1]),        # few heads: decode on the vector path
 ])
 def test_latent_attention_bf16_matrix_path_gpu(L, cuts):
     _latent_alone("cuda", L, 130, cuts=cuts, page=16, dtype=BF16, tol=0.03)
