@@ -25,6 +25,7 @@ import torch
 import torch.nn as nn
 
 from neuronx_distributed_inference_amd.models.model_base import DecoderModel
+from neuronx_distributed_inference_amd.modules.attention.attention_base import PHASE_CTE
 from neuronx_distributed_inference_amd.ops import seqmix
 
 
@@ -38,6 +39,9 @@ class LayerRun:
 
     def __call__(self, h, residual, cos, sin, kv_mgr, position_ids, phase,
                  attention_mask, seq_ids, **_):
+        # context encoding = every row starts its sequence in this step;
+        # mixers may take a whole-prompt path then
+        kv_mgr.step.fresh = phase == PHASE_CTE
         return self.layer(h, kv_mgr, self.run_idx), None
 
 

@@ -263,7 +263,7 @@ class SoputarLatentMixer(nn.Module):
         uk, uv = w(s + "uk"), w(s + "uv")
         C = uk.shape[1]
         out[d + "core.uk"] = uk.view(H, -1, C).contiguous()                   # (H, dim, C)
-        out[d + "core.uv_t"] = uv.view(H, -1, C).transpose(1, 2).contiguous()  # (H, C, vdim)
+        out[d + "core.uv"] = uv.view(H, -1, C).contiguous()                   # (H, vdim, C)
         out[d + "core.sink"] = f(s + "sink")
         out[d + "o_proj.weight"] = w(s + "o")
 

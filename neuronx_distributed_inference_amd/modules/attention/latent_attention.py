@@ -8,13 +8,19 @@ interleaved pair layout on the first ``rot_dims`` channels of the rotated
 part. The softmax denominator carries one extra term ``exp(sink_h)`` per
 head: a key without a value, unscaled.
 
-The engine computes this in the *absorbed* form, which never expands the
-cache: ``q_plain . (W_uk c) = (W_uk^T q_plain) . c``, so the query is mapped
-into latent space (one small batched GEMM per step), attention runs as
+Steps that continue a sequence (decoded tokens, later prompt portions, mixed
+batches) are computed in the *absorbed* form, which never expands the cache:
+``q_plain . (W_uk c) = (W_uk^T q_plain) . c``, so the query is mapped into
+latent space (one small batched GEMM per step), attention runs as
 multi-query attention over cache rows ``[c | k_rot]`` whose values are the
 rows' own first ``kv_rank`` channels, and ``W_uv`` is applied to the
 attended latent afterwards. One page row per token holds everything; there
-is no value cache.
+is no value cache. A step in which every row starts its sequence (a whole
+prompt, ``step.fresh``) has all its keys at hand and takes the *expanded*
+form instead: keys and values are materialised per head for the step only
+(two GEMMs) and ordinary multi-head attention runs over them, which costs
+``dim + rot_dim`` instead of ``kv_rank + rot_dim`` multiply-adds per score.
+The cache rows are written either way.
 
 The module owns the latent norm, the two up-projections, the sink and the
 cache access; the projections of the layer input (queries and the
@@ -47,12 +53,13 @@ class LatentSinkAttention(nn.Module):
         self.latent_norm = StreamRMSNorm(kv_rank, eps=eps, one_plus=False)
         self.register_buffer("inv_freq", interleaved_inv_freq(rope_base, rot_dims),
                              persistent=False)
-        # per-head up-projections, stored for the batched products:
-        # uk (H, dim, kv_rank): q_plain -> latent space;  uv_t (H, kv_rank, v_dim)
+        # per-head up-projections in checkpoint layout: uk (H, dim, kv_rank),
+        # uv (H, v_dim, kv_rank). Flattened they expand the latent; batched,
+        # uk maps q_plain into latent space and uv^T the attended latent out
         self.uk = nn.Parameter(torch.zeros(num_heads, dim, kv_rank, dtype=dtype),
                                requires_grad=False)
-        self.uv_t = nn.Parameter(torch.zeros(num_heads, kv_rank, v_dim, dtype=dtype),
-                                 requires_grad=False)
+        self.uv = nn.Parameter(torch.zeros(num_heads, v_dim, kv_rank, dtype=dtype),
+                               requires_grad=False)
         self.sink = nn.Parameter(torch.zeros(num_heads, dtype=torch.float32),
                                  requires_grad=False) if sink else None
 
@@ -77,8 +84,10 @@ class LatentSinkAttention(nn.Module):
         kc, _ = kv_mgr.get_cache(cache_idx)
         seqmix.paged_kv_write(kc.data, None, row.view(T, self.row), None,
                               kv_mgr.slot_mapping, step)
-        # query in latent space: [uk_h^T q_plain | rotated q_rot] per head
         q4 = q.unflatten(-1, (H, D + R))
+        if getattr(step, "fresh", False):
+            return self._expanded(q4, row, step)
+        # query in latent space: [uk_h^T q_plain | rotated q_rot] per head
         qa = torch.empty(B, S, H, self.row, dtype=dt, device=q.device)
         torch.bmm(q4[..., :D].flatten(0, 1).transpose(0, 1), self.uk,
                   out=qa.view(T, H, self.row)[..., :C].transpose(0, 1))
@@ -88,6 +97,25 @@ class LatentSinkAttention(nn.Module):
             qa.view(B, S, H * self.row), k_cache, k_cache[..., :C], step, kv_mgr.block_table,
             self.scale, H, sink=self.sink, out_dtype=dt)              # (B,S,H*C)
         out = torch.empty(B, S, H * self.v_dim, dtype=dt, device=q.device)
-        torch.bmm(lat.view(T, H, C).transpose(0, 1), self.uv_t,
+        torch.bmm(lat.view(T, H, C).transpose(0, 1), self.uv.transpose(1, 2),
                   out=out.view(T, H, self.v_dim).transpose(0, 1))
         return out
+
+    def _expanded(self, q4: torch.Tensor, row: torch.Tensor, step) -> torch.Tensor:
+        """Whole prompts: per-head keys [W_uk c | k_rot] and values W_uv c of
+        this step's tokens, attended in place: the (B, S) token grid is
+        addressed as B pages of S tokens."""
+        B, S, H = q4.shape[0], q4.shape[1], self.num_heads
+        D, R, C, Dv = self.dim, self.rot_dim, self.kv_rank, self.v_dim
+        dt = q4.dtype
+        c = row[..., :C]
+        kx = torch.empty(B, S, H, D + R, dtype=dt, device=q4.device)
+        kx[..., :D] = torch.nn.functional.linear(c, self.uk.view(H * D, C)).view(B, S, H, D)
+        kx[..., D:] = row[..., C:].unsqueeze(2)
+        vx = torch.nn.functional.linear(c, self.uv.view(H * Dv, C)).view(B, S, H, Dv)
+        qx = q4.clone(memory_format=torch.contiguous_format)
+        seqmix.rotate_interleaved(qx[..., D:], step, self.inv_freq, out=qx[..., D:])
+        pages = torch.arange(B, device=q4.device, dtype=torch.int32).view(B, 1)
+        return seqmix.paged_attention(
+            qx.view(B, S, H * (D + R)), kx, vx, step, pages, self.scale, H,
+            sink=self.sink, out_dtype=dt)

@@ -686,39 +686,66 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
 #pragma unroll
     for (int nb = 0; nb < DVP / 16; ++nb) o_acc[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
+    // a tile's K and V lines travel global -> registers -> LDS; the next tile's
+    // loads are issued before the current tile's products, so their latency
+    // (block-table lookup, then the line) hides behind the matrix work
+    constexpr int NKI = (MA_KT * (DKP / 8) + 255) / 256;
+    constexpr int NVI = (MA_KT * (DVP / 8) + 255) / 256;
+    uint4 rk[NKI], rv[NVI];
+#define MA_FETCH(BASE)                                                                     \
+    {                                                                                      \
+        _Pragma("unroll") for (int x = 0; x < NKI; ++x) {                                  \
+            const int c = tid + x * 256;                                                   \
+            const int m = c / (DKP / 8), part = c % (DKP / 8);                             \
+            uint4 raw = make_uint4(0, 0, 0, 0);                                            \
+            if (c < MA_KT * (DKP / 8) && (BASE) + m < n && part * 8 < Dk) {                \
+                const int mm = (BASE) + m;                                                 \
+                const int j = mm < nfirst ? mm : lo + (mm - nfirst);                       \
+                const int blk = bt[j / bsz];                                               \
+                const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);             \
+                raw = *reinterpret_cast<const uint4*>(kc + slot * ktok + (long)g * khead + part * 8); \
+            }                                                                              \
+            rk[x] = raw;                                                                   \
+        }                                                                                  \
+        _Pragma("unroll") for (int x = 0; x < NVI; ++x) {                                  \
+            const int c = tid + x * 256;                                                   \
+            const int m = c % MA_KT, part = c / MA_KT;   /* consecutive lanes: consecutive keys */ \
+            uint4 raw = make_uint4(0, 0, 0, 0);                                            \
+            if (c < MA_KT * (DVP / 8) && (BASE) + m < n && part * 8 < dvn) {               \
+                const int mm = (BASE) + m;                                                 \
+                const int j = mm < nfirst ? mm : lo + (mm - nfirst);                       \
+                const int blk = bt[j / bsz];                                               \
+                const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);             \
+                raw = *reinterpret_cast<const uint4*>(vc + slot * vtok + (long)g * vhead + dv0 + \
+                                                      part * 8);                           \
+            }                                                                              \
+            rv[x] = raw;                                                                   \
+        }                                                                                  \
+    }
+    MA_FETCH(0)
     for (int base = 0; base < n; base += MA_KT) {
-        // ---- stage K (row-major) and V (transposed) tiles
-        for (int c = tid; c < MA_KT * (DKP / 8); c += 256) {
-            const int m = c / (DKP / 8), part = c % (DKP / 8);
-            uint4 raw = make_uint4(0, 0, 0, 0);
-            if (base + m < n && part * 8 < Dk) {
-                const int mm = base + m;
-                const int j = mm < nfirst ? mm : lo + (mm - nfirst);
-                const int blk = bt[j / bsz];
-                const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
-                raw = *reinterpret_cast<const uint4*>(kc + slot * ktok + (long)g * khead + part * 8);
-            }
-            *reinterpret_cast<uint4*>(k_lds + m * KS + part * 8) = raw;
-        }
-        for (int c = tid; c < MA_KT * (DVP / 8); c += 256) {
-            const int m = c % MA_KT, part = c / MA_KT;   // consecutive lanes: consecutive keys
-            uint4 raw = make_uint4(0, 0, 0, 0);
-            if (base + m < n && part * 8 < dvn) {
-                const int mm = base + m;
-                const int j = mm < nfirst ? mm : lo + (mm - nfirst);
-                const int blk = bt[j / bsz];
-                const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
-                raw = *reinterpret_cast<const uint4*>(vc + slot * vtok + (long)g * vhead + dv0 +
-                                                      part * 8);
-            }
-            const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+        // ---- registers -> LDS: K row-major, V transposed
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                vt_lds[(part * 8 + 2 * e) * VS + m] = (uint16_t)(u[e] & 0xffffu);
-                vt_lds[(part * 8 + 2 * e + 1) * VS + m] = (uint16_t)(u[e] >> 16);
+        for (int x = 0; x < NKI; ++x) {
+            const int c = tid + x * 256;
+            if (c < MA_KT * (DKP / 8))
+                *reinterpret_cast<uint4*>(k_lds + (c / (DKP / 8)) * KS + (c % (DKP / 8)) * 8) = rk[x];
+        }
+#pragma unroll
+        for (int x = 0; x < NVI; ++x) {
+            const int c = tid + x * 256;
+            if (c < MA_KT * (DVP / 8)) {
+                const int m = c % MA_KT, part = c / MA_KT;
+                const uint32_t u[4] = {rv[x].x, rv[x].y, rv[x].z, rv[x].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    vt_lds[(part * 8 + 2 * e) * VS + m] = (uint16_t)(u[e] & 0xffffu);
+                    vt_lds[(part * 8 + 2 * e + 1) * VS + m] = (uint16_t)(u[e] >> 16);
+                }
             }
         }
         __syncthreads();
+        if (base + MA_KT < n) MA_FETCH(base + MA_KT)     // in flight during the products below
         // ---- S^T = K Q^T: lane gets keys 16*kb + 4*lg + r of its own row lr
         float sv[KB][4];
         float mt = -INFINITY;
@@ -802,6 +829,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         }
         __syncthreads();
     }
+#undef MA_FETCH
     // ---- epilogue: rows 4*lg + r of this wave, channel 16*nb + lr. A sink adds
     // one term to the row's denominator (computed by the lane that owns the row)
     float fin = l_run > 0.f ? 1.f / l_run : 0.f;

@@ -158,6 +158,8 @@ class StepLayout:
         # the residual stream in the GEMM input dtype, handed from one
         # sublayer's residual kernel to the next sublayer (None: not yet made)
         self.stream_copy = None
+        # True when every row of the step starts its sequence (a whole prompt)
+        self.fresh = False
 
     def i32(self, t: torch.Tensor) -> torch.Tensor:
         """int32 copy of a per-step index tensor (block table, slot mapping),

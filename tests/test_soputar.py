@@ -375,7 +375,8 @@ def test_capped_attention_bf16_matrix_path_gpu(L, cuts):
 
 
 # ------------------------------------------------------------ latent attention
-def _latent_alone(device, L, T, cuts=None, page=4, dtype=F32, tol=3e-5, sink=None, spikes=()):
+def _latent_alone(device, L, T, cuts=None, page=4, dtype=F32, tol=3e-5, sink=None, spikes=(),
+                  fresh=False):
     torch.manual_seed(5)
     Wd = 14
     H, D, R, Dv, C = L["heads"], L["dim"], L["rot_dim"], L["vdim"], L["kv_rank"]
@@ -401,7 +402,7 @@ def _latent_alone(device, L, T, cuts=None, page=4, dtype=F32, tol=3e-5, sink=Non
                               L["rot"]["dims"], dtype)
     att.latent_norm.weight.data = W["p.dkv.norm"].float()
     att.uk.data = W["p.uk"].view(H, D, C).to(dtype)
-    att.uv_t.data = W["p.uv"].view(H, Dv, C).transpose(1, 2).contiguous().to(dtype)
+    att.uv.data = W["p.uv"].view(H, Dv, C).to(dtype)
     att.sink.data = W["p.sink"].float()
     att = att.to(device)
     nblk = (T + page - 1) // page
@@ -416,6 +417,7 @@ def _latent_alone(device, L, T, cuts=None, page=4, dtype=F32, tol=3e-5, sink=Non
         pos = torch.arange(at, at + n).view(1, n).to(device)
         mgr.set_step_context(bt, generate_slot_mapping(bt, pos, page))
         st = seqmix.StepLayout(pos, torch.zeros(1, dtype=torch.long, device=device))
+        st.fresh = fresh and at == 0          # whole-prompt form for the first portion
         sl = slice(at, at + n)
         y = att(q[sl].view(1, n, -1).to(device, dtype), dkv[sl].view(1, n, -1).to(device, dtype),
                 mgr, 0, st)
@@ -436,6 +438,15 @@ def test_latent_attention_portions(device, L):
     _latent_alone(device, L, 26)
     _latent_alone(device, L, 26, cuts=[1, 2, 7, 1, 1, 1, 13])
     _latent_alone(device, L, 26, cuts=[3] + [1] * 23, page=8)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("L", [latent_cfg(), latent_cfg(2, 6, 8, 10, 12, base=9.0, dims=4)])
+def test_latent_attention_whole_prompt_form(device, L):
+    """A prompt taken in the expanded form, then continued from the cache
+    rows it left (absorbed form): both equal the oracle."""
+    _latent_alone(device, L, 26, fresh=True)
+    _latent_alone(device, L, 26, cuts=[17, 1, 1, 7], fresh=True)
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -470,6 +481,7 @@ def test_latent_attention_far_keys_and_positions(device, cuts):
 ])
 def test_latent_attention_bf16_matrix_path_gpu(L, cuts):
     _latent_alone("cuda", L, 130, cuts=cuts, page=16, dtype=BF16, tol=0.03)
+    _latent_alone("cuda", L, 130, cuts=[100] + [1] * 30, page=16, dtype=BF16, tol=0.03, fresh=True)
 
 
 # ------------------------------------------------------------------ delta rule
