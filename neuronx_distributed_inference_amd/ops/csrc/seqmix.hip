@@ -620,7 +620,7 @@ DEV uint16_t f2bf_rne(float f) {
     return (uint16_t)(u >> 16);
 }
 
-template <int DKP, int DVP, int MA_KT>
+template <int DKP, int DVP, int MA_KT, bool PREFETCH>
 __global__ void __launch_bounds__(256)
 paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __restrict__ kc,
                        const bf16* __restrict__ vc, const int* __restrict__ pos,
@@ -686,9 +686,10 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
 #pragma unroll
     for (int nb = 0; nb < DVP / 16; ++nb) o_acc[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    // a tile's K and V lines travel global -> registers -> LDS; the next tile's
-    // loads are issued before the current tile's products, so their latency
-    // (block-table lookup, then the line) hides behind the matrix work
+    // a tile's K and V lines travel global -> registers -> LDS. With PREFETCH
+    // (wide rows: one workgroup per CU, nothing else to hide latency) the next
+    // tile's loads are issued before the current tile's products; without, the
+    // registers are reused and more workgroups share a CU
     constexpr int NKI = (MA_KT * (DKP / 8) + 255) / 256;
     constexpr int NVI = (MA_KT * (DVP / 8) + 255) / 256;
     uint4 rk[NKI], rv[NVI];
@@ -722,8 +723,9 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
             rv[x] = raw;                                                                   \
         }                                                                                  \
     }
-    MA_FETCH(0)
+    if constexpr (PREFETCH) MA_FETCH(0)
     for (int base = 0; base < n; base += MA_KT) {
+        if constexpr (!PREFETCH) MA_FETCH(base)
         // ---- registers -> LDS: K row-major, V transposed
 #pragma unroll
         for (int x = 0; x < NKI; ++x) {
@@ -745,7 +747,9 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
             }
         }
         __syncthreads();
-        if (base + MA_KT < n) MA_FETCH(base + MA_KT)     // in flight during the products below
+        if constexpr (PREFETCH) {
+            if (base + MA_KT < n) MA_FETCH(base + MA_KT) // in flight during the products below
+        }
         // ---- S^T = K Q^T: lane gets keys 16*kb + 4*lg + r of its own row lr
         float sv[KB][4];
         float mt = -INFINITY;
@@ -856,6 +860,242 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
             if (gp) o *= sigmoidf_(__bfloat162float(gp[d]));
             op[d] = __float2bfloat16(o);
         }
+    }
+}
+
+// ------------------------------------ latent-cache decode, matrix cores
+// Single-token steps of multi-query layers whose values are the first Dv
+// channels of the (one) key row per token — the absorbed form of latent
+// attention: 16 query heads of one token are the 16 rows of the score tile.
+// All four waves compute the (cheap) scores of a 32-key tile; wave w owns value
+// channels [128w, 128w+128), so a workgroup covers 512 of them and the key row
+// is fetched from memory once: global -> registers (next tile prefetched) -> LDS
+// row-major, then V^T is cut out of that LDS tile. Causal, optional sink.
+// Grid: (tokens x key splits, head chunks of 16 x value splits of 512, batch
+// rows). With nks > 1 key splits a workgroup scans every nks-th run of tiles and
+// leaves an unnormalised partial (fp32 values, running max, sum) in `ws`;
+// latent_decode_merge_kernel folds the splits and the sink.
+#define LD_KT 32
+#define LD_VW 128                            // value channels per wave
+
+template <int DKP>
+__global__ void __launch_bounds__(256)
+latent_decode_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __restrict__ kc,
+                          long ktok, const int* __restrict__ pos, const int* __restrict__ seq,
+                          const int* __restrict__ btab, int max_blocks,
+                          const float* __restrict__ sink, bf16* __restrict__ out, int H, int Dk,
+                          int Dv, int bsz, int S, float scale, int nsplit, int nks,
+                          float* __restrict__ ws) {
+    constexpr int KS = DKP + 8;
+    constexpr int VS = LD_KT + 8;
+    constexpr int VCH = 4 * LD_VW;
+    extern __shared__ __attribute__((aligned(16))) uint16_t ld_lds[];
+    uint16_t* k_lds = ld_lds;                            // LD_KT * KS
+    uint16_t* vt_lds = ld_lds + LD_KT * KS;              // VCH * VS
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
+    const int b = blockIdx.z, t = blockIdx.x / nks, ksp = blockIdx.x % nks;
+    const int h0 = (blockIdx.y / nsplit) * 16;
+    const int dv0 = (blockIdx.y % nsplit) * VCH;         // this workgroup's first value channel
+    const int dvn = min(VCH, Dv - dv0);
+    if (seq[b] < 0) return;
+    const int p = pos[(long)b * S + t];
+    if (p < 0) return;                                   // uniform
+    const int h = h0 + lr;                               // this lane's query row
+    const bool hv = h < H;
+    bf16x8_t qf[DKP / 32];
+    {
+        const bf16* qp = q + ((long)b * S + t) * qstride + (long)h * Dk;
+#pragma unroll
+        for (int ks = 0; ks < DKP / 32; ++ks) {
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (hv && ks * 32 + lg * 8 < Dk) raw = *reinterpret_cast<const uint4*>(qp + ks * 32 + lg * 8);
+            qf[ks] = *reinterpret_cast<bf16x8_t*>(&raw);
+        }
+    }
+    const int* bt = btab + (long)b * max_blocks;
+    // this split's keys [k_lo, n): a contiguous run of 32-key tiles
+    const int tiles = (p + 1 + LD_KT - 1) / LD_KT, per = (tiles + nks - 1) / nks;
+    const int k_lo = ksp * per * LD_KT;
+    const int n = min(p + 1, (ksp + 1) * per * LD_KT);
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4_t o_acc[LD_VW / 16];
+#pragma unroll
+    for (int nb = 0; nb < LD_VW / 16; ++nb) o_acc[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    constexpr int NKI = (LD_KT * (DKP / 8) + 255) / 256;
+    uint4 rk[NKI];
+#define LD_FETCH(BASE)                                                                     \
+    _Pragma("unroll") for (int x = 0; x < NKI; ++x) {                                      \
+        const int c = tid + x * 256;                                                       \
+        const int m = c / (DKP / 8), part = c % (DKP / 8);                                 \
+        uint4 raw = make_uint4(0, 0, 0, 0);                                                \
+        if (c < LD_KT * (DKP / 8) && (BASE) + m < n && part * 8 < Dk) {                    \
+            const int j = (BASE) + m;                                                      \
+            const int blk = bt[j / bsz];                                                   \
+            const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);                 \
+            raw = *reinterpret_cast<const uint4*>(kc + slot * ktok + part * 8);            \
+        }                                                                                  \
+        rk[x] = raw;                                                                       \
+    }
+    LD_FETCH(k_lo)
+    for (int base = k_lo; base < n; base += LD_KT) {
+#pragma unroll
+        for (int x = 0; x < NKI; ++x) {
+            const int c = tid + x * 256;
+            if (c < LD_KT * (DKP / 8))
+                *reinterpret_cast<uint4*>(k_lds + (c / (DKP / 8)) * KS + (c % (DKP / 8)) * 8) = rk[x];
+        }
+        __syncthreads();
+        if (base + LD_KT < n) LD_FETCH(base + LD_KT)     // in flight during the work below
+        // ---- V^T (channels dv0..dv0+dvn) out of the K tile
+        for (int c = tid; c < LD_KT * (VCH / 8); c += 256) {
+            const int m = c % LD_KT, part = c / LD_KT;
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (part * 8 < dvn) raw = *reinterpret_cast<const uint4*>(k_lds + m * KS + dv0 + part * 8);
+            const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                vt_lds[(part * 8 + 2 * e) * VS + m] = (uint16_t)(u[e] & 0xffffu);
+                vt_lds[(part * 8 + 2 * e + 1) * VS + m] = (uint16_t)(u[e] >> 16);
+            }
+        }
+        // ---- S^T = K Q^T: lane gets keys 16*kb + 4*lg + r of row lr
+        float sv[2][4];
+        float mt = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < DKP / 32; ++ks) {
+                const bf16x8_t ka = *reinterpret_cast<const bf16x8_t*>(
+                    k_lds + (kb * 16 + lr) * KS + ks * 32 + lg * 8);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[ks], acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int j = base + kb * 16 + lg * 4 + r;
+                const float x = (j < n && hv) ? acc[r] * scale : -INFINITY;
+                sv[kb][r] = x;
+                mt = fmaxf(mt, x);
+            }
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 16, WAVE));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, WAVE));
+        const float m_new = fmaxf(m_run, mt);
+        float corr = 1.f, psum = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float pv = (m_new > -INFINITY && sv[kb][r] > -INFINITY)
+                    ? expf(sv[kb][r] - m_new) : 0.f;
+                sv[kb][r] = pv;
+                psum += pv;
+            }
+        if (m_new > -INFINITY) corr = expf(m_run - m_new);
+        psum += __shfl_xor(psum, 16, WAVE);
+        psum += __shfl_xor(psum, 32, WAVE);
+        l_run = l_run * corr + psum;
+        m_run = m_new;
+        float cr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, lg * 4 + r, WAVE);
+#pragma unroll
+        for (int nb = 0; nb < LD_VW / 16; ++nb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o_acc[nb][r] *= cr[r];
+        __syncthreads();                                 // V^T complete
+        // ---- O += P V for this wave's 128 channels, P as hi + lo
+        {
+            union { bf16x8_t v; uint16_t u[8]; } ph, pl;
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) {
+                const float pv = sv[jj >> 2][jj & 3];
+                const uint16_t hb = f2bf_rne(pv);
+                ph.u[jj] = hb;
+                pl.u[jj] = f2bf_rne(pv - __uint_as_float((uint32_t)hb << 16));
+            }
+#pragma unroll
+            for (int nb = 0; nb < LD_VW / 16; ++nb) {
+                union { bf16x8_t v; uint2 h2[2]; } vb;
+                const uint16_t* vp = vt_lds + (wv * LD_VW + nb * 16 + lr) * VS + 4 * lg;
+                vb.h2[0] = *reinterpret_cast<const uint2*>(vp);
+                vb.h2[1] = *reinterpret_cast<const uint2*>(vp + 16);
+                o_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph.v, vb.v, o_acc[nb], 0, 0, 0);
+                o_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl.v, vb.v, o_acc[nb], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+#undef LD_FETCH
+    if (nks > 1) {
+        // partial result: [(token, head, split)][Dv values | max | sum]
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int hh = h0 + lg * 4 + r;
+            const float mr = __shfl(m_run, lg * 4 + r, WAVE), lrn = __shfl(l_run, lg * 4 + r, WAVE);
+            if (hh >= H) continue;
+            float* wp = ws + ((((long)b * S + t) * H + hh) * nks + ksp) * (long)(Dv + 2);
+#pragma unroll
+            for (int nb = 0; nb < LD_VW / 16; ++nb) {
+                const int d = wv * LD_VW + nb * 16 + lr;
+                if (d < dvn) wp[dv0 + d] = o_acc[nb][r];
+            }
+            if (dv0 == 0 && wv == 0 && lr == 0) { wp[Dv] = mr; wp[Dv + 1] = lrn; }
+        }
+        return;
+    }
+    float fin = l_run > 0.f ? 1.f / l_run : 0.f;
+    if (sink && hv) {
+        const float sk = sink[h];
+        const float mf = fmaxf(m_run, sk);
+        const float ca = m_run > -INFINITY ? expf(m_run - mf) : 0.f;
+        fin = ca / (l_run * ca + expf(sk - mf));
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int hh = h0 + lg * 4 + r;
+        const float inv = __shfl(fin, lg * 4 + r, WAVE);
+        if (hh >= H) continue;
+        bf16* op = out + (((long)b * S + t) * H + hh) * (long)Dv + dv0 + wv * LD_VW;
+#pragma unroll
+        for (int nb = 0; nb < LD_VW / 16; ++nb) {
+            const int d = wv * LD_VW + nb * 16 + lr;
+            if (d < dvn) op[nb * 16 + lr] = __float2bfloat16(o_acc[nb][r] * inv);
+        }
+    }
+}
+
+// one wave per (token, head): out = sum_i o_i e^(m_i - M) / (sum_i l_i e^(m_i - M)
+// + e^(sink - M)), M the largest of the splits' maxima and the sink
+__global__ void latent_decode_merge_kernel(const float* __restrict__ ws,
+                                           const float* __restrict__ sink,
+                                           const int* __restrict__ pos, const int* __restrict__ seq,
+                                           bf16* __restrict__ out, long ntok, int S, int H, int Dv,
+                                           int nks) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const long wid = (long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (wid >= ntok * H) return;
+    const long tok = wid / H;
+    const int h = wid % H;
+    if (pos[tok] < 0 || seq[tok / S] < 0) return;
+    const float* wp = ws + wid * nks * (long)(Dv + 2);
+    const float sk = sink ? sink[h] : -INFINITY;
+    float M = sk;
+    for (int i = 0; i < nks; ++i) M = fmaxf(M, wp[i * (long)(Dv + 2) + Dv]);
+    float L = sink ? expf(sk - M) : 0.f;
+    for (int i = 0; i < nks; ++i) {
+        const float mi = wp[i * (long)(Dv + 2) + Dv];
+        if (mi > -INFINITY) L += wp[i * (long)(Dv + 2) + Dv + 1] * expf(mi - M);
+    }
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+    for (int d = lane; d < Dv; d += WAVE) {
+        float o = 0.f;
+        for (int i = 0; i < nks; ++i) {
+            const float mi = wp[i * (long)(Dv + 2) + Dv];
+            if (mi > -INFINITY) o += wp[i * (long)(Dv + 2) + d] * expf(mi - M);
+        }
+        out[wid * Dv + d] = __float2bfloat16(o * inv);
     }
 }
 
@@ -1375,7 +1615,7 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
                   const float* sink, const void* gate, long gstride, void* out, int io_bf16,
                   int out_bf16, int B, int S, int H, int G, int Dk, int Dv, int bsz,
                   float scale, int window, int keep, float cap, float qt_coef, int qt_every,
-                  hipStream_t st) {
+                  float* ws, int nks, hipStream_t st) {
     if ((long)B * S <= 0) return 0;
     if (Dv > WAVE * 8 || H % G != 0 || Dk <= 0 || Dv <= 0) return -1;
     if (!io_bf16 && out_bf16) return -2;
@@ -1386,6 +1626,39 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
                       ((uintptr_t)kc % 16) == 0;
     const bool v_al = (Dv % 8) == 0 && (vtok % vecn) == 0 && (vhead % vecn) == 0 &&
                       ((uintptr_t)vc % 16) == 0;
+    if (io_bf16 && out_bf16 && S == 1 && G == 1 && vc == kc && vtok == ktok && k_al && v_al &&
+        !r1 && !gate && cap <= 0.f && qt_every <= 0 && window == 0x7fffffff && H >= 8 &&
+        Dk <= 640 && (qstride % 8) == 0 && ((uintptr_t)q % 16) == 0) {
+        // latent caches, single-token steps: one workgroup per token reads each
+        // key row once and covers 512 value channels
+        const int dkp = (Dk + 31) & ~31;
+        const int nsplit = (Dv + 511) / 512, hch = (H + 15) / 16;
+        if (nks < 1 || !ws) nks = 1;
+        dim3 gl(S * nks, hch * nsplit, B), bl(256);
+#define LD(DKV) do { \
+            const size_t lsh = (size_t)(LD_KT * (DKV + 8) + 4 * LD_VW * (LD_KT + 8)) * 2; \
+            static bool attr_set = false; \
+            if (!attr_set) { \
+                if (hipFuncSetAttribute((const void*)latent_decode_mfma_kernel<DKV>, \
+                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lsh) != hipSuccess) return -5; \
+                attr_set = true; \
+            } \
+            latent_decode_mfma_kernel<DKV><<<gl, bl, lsh, st>>>( \
+                (const bf16*)q, qstride, (const bf16*)kc, ktok, pos, seq, btab, max_blocks, sink, \
+                (bf16*)out, H, Dk, Dv, bsz, S, scale, nsplit, nks, ws); } while (0)
+        if (dkp <= 128) LD(128);
+        else if (dkp <= 256) LD(256);
+        else if (dkp <= 384) LD(384);
+        else if (dkp <= 576) LD(576);
+        else LD(640);
+#undef LD
+        if (nks > 1) {
+            const long waves = (long)B * S * H;
+            latent_decode_merge_kernel<<<(unsigned)((waves + 3) / 4), 4 * WAVE, 0, st>>>(
+                ws, sink, pos, seq, (bf16*)out, (long)B * S, S, H, Dv, nks);
+        }
+        return (int)hipGetLastError();
+    }
     {
         // matrix-core path: bf16 steps with prompt portions (any head sizes in
         // multiples of 8: keys up to 640 wide, wide values split over
@@ -1402,7 +1675,7 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
             const int QTm = MA_ROWS / rp;
             const int nsplit = wide ? (Dv + 127) / 128 : 1;
             dim3 gm((S + QTm - 1) / QTm, G * nsplit, B), bm(256);
-#define MA(DKV, DVV, KTV) paged_attn_mfma_kernel<DKV, DVV, KTV><<<gm, bm, 0, st>>>( \
+#define MA(DKV, DVV, KTV) paged_attn_mfma_kernel<DKV, DVV, KTV, (KTV == 32)><<<gm, bm, 0, st>>>( \
         (const bf16*)q, qstride, (const bf16*)kc, (const bf16*)vc, pos, seq, btab, max_blocks, \
         r1, r2, (const bf16*)gate, gstride, (bf16*)out, H, G, Dk, Dv, bsz, S, scale, window, \
         keep, QTm, ktok, khead, vtok, vhead, sink, cap, qt_coef, qt_every, nsplit)

@@ -269,6 +269,16 @@ def paged_attention(q, k_cache, v_cache, step: StepLayout, block_table, scale: f
         assert v_cache.stride(0) == v_cache.stride(1) * v_cache.shape[1]
         assert k_cache.dtype == v_cache.dtype == q.dtype
         coef, every = (0.0, 0) if q_temp is None else (float(q_temp[0]), int(q_temp[1]))
+        # single-token steps over latent caches (values inside the one key
+        # row): few workgroups per step, so the keys are split over several
+        # and merged; the partials need a workspace
+        ws, nks = None, 1
+        if S == 1 and G == 1 and q.dtype == torch.bfloat16 and \
+                v_cache.data_ptr() == k_cache.data_ptr() and window is None:
+            groups = B * ((H + 15) // 16) * ((Dv + 511) // 512)
+            nks = max(1, min(8, 256 // max(groups, 1), (bt.shape[1] * k_cache.shape[1]) // 128))
+            if nks > 1:
+                ws = torch.empty(B * H * nks * (Dv + 2), dtype=torch.float32, device=q.device)
         _check(lib.nx_paged_attn(
             _p(q), ctypes.c_long(_rows_view(q)), _p(k_cache), ctypes.c_long(k_cache.stride(1)),
             ctypes.c_long(k_cache.stride(2)), _p(v_cache), ctypes.c_long(v_cache.stride(1)),
@@ -281,7 +291,7 @@ def paged_attention(q, k_cache, v_cache, step: StepLayout, block_table, scale: f
             k_cache.shape[1], ctypes.c_float(scale),
             int(window) if window is not None else 0x7fffffff, int(keep_first),
             ctypes.c_float(softcap or 0.0), ctypes.c_float(coef), every,
-            _stream()), "paged_attention")
+            _p(ws), nks, _stream()), "paged_attention")
         return out
     return ref.paged_attention(
         q.reshape(B, S, H, Dk), k_cache, v_cache, step.positions, block_table, scale,

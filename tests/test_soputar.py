@@ -484,6 +484,16 @@ def test_latent_attention_bf16_matrix_path_gpu(L, cuts):
     _latent_alone("cuda", L, 130, cuts=[100] + [1] * 30, page=16, dtype=BF16, tol=0.03, fresh=True)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("L", [latent_cfg(16, 64, 64, 64, 512, scale=0.07),
+                               latent_cfg(20, 32, 32, 48, 224, scale=0.1)])
+def test_latent_attention_decode_key_splits_gpu(L):
+    """Long contexts split a decoded token's keys over several workgroups
+    whose partial softmaxes are merged (sink included once)."""
+    _latent_alone("cuda", L, 420, cuts=[400] + [1] * 20, page=16, dtype=BF16, tol=0.03)
+    _latent_alone("cuda", L, 300, cuts=[290] + [1] * 10, page=16, dtype=BF16, tol=0.03, sink=3.0)
+
+
 # ------------------------------------------------------------------ delta rule
 def _delta_alone(device, R, T, cuts, slots=(1,)):
     torch.manual_seed(4)
