@@ -725,8 +725,41 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
     }
     if constexpr (PREFETCH) MA_FETCH(0)
     for (int base = 0; base < n; base += MA_KT) {
-        if constexpr (!PREFETCH) MA_FETCH(base)
-        // ---- registers -> LDS: K row-major, V transposed
+        if constexpr (!PREFETCH) {
+            // ---- global -> LDS directly: K row-major, V transposed
+            for (int c = tid; c < MA_KT * (DKP / 8); c += 256) {
+                const int m = c / (DKP / 8), part = c % (DKP / 8);
+                uint4 raw = make_uint4(0, 0, 0, 0);
+                if (base + m < n && part * 8 < Dk) {
+                    const int mm = base + m;
+                    const int j = mm < nfirst ? mm : lo + (mm - nfirst);
+                    const int blk = bt[j / bsz];
+                    const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
+                    raw = *reinterpret_cast<const uint4*>(kc + slot * ktok + (long)g * khead + part * 8);
+                }
+                *reinterpret_cast<uint4*>(k_lds + m * KS + part * 8) = raw;
+            }
+            for (int c = tid; c < MA_KT * (DVP / 8); c += 256) {
+                const int m = c % MA_KT, part = c / MA_KT;   // consecutive lanes: consecutive keys
+                uint4 raw = make_uint4(0, 0, 0, 0);
+                if (base + m < n && part * 8 < dvn) {
+                    const int mm = base + m;
+                    const int j = mm < nfirst ? mm : lo + (mm - nfirst);
+                    const int blk = bt[j / bsz];
+                    const long slot = (long)(blk < 0 ? 0 : blk) * bsz + (j % bsz);
+                    raw = *reinterpret_cast<const uint4*>(vc + slot * vtok + (long)g * vhead + dv0 +
+                                                          part * 8);
+                }
+                const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    vt_lds[(part * 8 + 2 * e) * VS + m] = (uint16_t)(u[e] & 0xffffu);
+                    vt_lds[(part * 8 + 2 * e + 1) * VS + m] = (uint16_t)(u[e] >> 16);
+                }
+            }
+        }
+        // ---- (prefetched) registers -> LDS
+        if constexpr (PREFETCH) {
 #pragma unroll
         for (int x = 0; x < NKI; ++x) {
             const int c = tid + x * 256;
@@ -745,6 +778,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
                     vt_lds[(part * 8 + 2 * e + 1) * VS + m] = (uint16_t)(u[e] >> 16);
                 }
             }
+        }
         }
         __syncthreads();
         if constexpr (PREFETCH) {
@@ -1089,13 +1123,18 @@ __global__ void latent_decode_merge_kernel(const float* __restrict__ ws,
         if (mi > -INFINITY) L += wp[i * (long)(Dv + 2) + Dv + 1] * expf(mi - M);
     }
     const float inv = L > 0.f ? 1.f / L : 0.f;
+    float wgt[8];                                        // nks <= 8
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float mi = i < nks ? wp[i * (long)(Dv + 2) + Dv] : -INFINITY;
+        wgt[i] = mi > -INFINITY ? expf(mi - M) * inv : 0.f;
+    }
     for (int d = lane; d < Dv; d += WAVE) {
         float o = 0.f;
-        for (int i = 0; i < nks; ++i) {
-            const float mi = wp[i * (long)(Dv + 2) + Dv];
-            if (mi > -INFINITY) o += wp[i * (long)(Dv + 2) + d] * expf(mi - M);
-        }
-        out[wid * Dv + d] = __float2bfloat16(o * inv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (i < nks) o += wp[i * (long)(Dv + 2) + d] * wgt[i];
+        out[wid * Dv + d] = __float2bfloat16(o);
     }
 }
 
@@ -1634,6 +1673,7 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
         const int dkp = (Dk + 31) & ~31;
         const int nsplit = (Dv + 511) / 512, hch = (H + 15) / 16;
         if (nks < 1 || !ws) nks = 1;
+        if (nks > 8) return -6;
         dim3 gl(S * nks, hch * nsplit, B), bl(256);
 #define LD(DKV) do { \
             const size_t lsh = (size_t)(LD_KT * (DKV + 8) + 4 * LD_VW * (LD_KT + 8)) * 2; \
