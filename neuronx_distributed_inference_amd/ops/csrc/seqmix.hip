@@ -1445,7 +1445,80 @@ __global__ void gelu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ ou
 
 // ------------------------------------------------------------------ RMS norm
 // x / sqrt(mean(x^2) + eps) * w (or * (1 + w)); one 256-thread workgroup per
-// row, fp32 statistics; input and output rows may be strided slices
+// row, fp32 statistics; input and output rows may be strided slices. The *_vec
+// variants move 8 channels per thread with 16-byte accesses (widths that are
+// multiples of 8 on 16-byte aligned rows); the second pass re-reads the row
+// from cache, so any width works.
+template <typename T> DEV void store8(T* p, const float* v);
+template <> DEV void store8<float>(float* p, const float* v) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+template <> DEV void store8<bf16>(bf16* p, const float* v) {
+    uint32_t pk[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        pk[e] = (uint32_t)f2bf_rne(v[2 * e]) | ((uint32_t)f2bf_rne(v[2 * e + 1]) << 16);
+    *reinterpret_cast<uint4*>(p) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+}
+
+template <typename TIn, typename TOut>
+__global__ void __launch_bounds__(LN_THREADS)
+rms_norm_vec_kernel(const TIn* __restrict__ x, long xs, const float* __restrict__ w, int one_plus,
+                    float eps, TOut* __restrict__ out, long os, int C) {
+    __shared__ float red[LN_THREADS / WAVE];
+    const long row = blockIdx.x;
+    const TIn* xr = x + row * xs;
+    float s = 0.f;
+    for (int c = threadIdx.x * 8; c < C; c += LN_THREADS * 8) {
+        float v[8];
+        load8<TIn>(xr + c, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s += v[e] * v[e];
+    }
+    const float inv = 1.f / sqrtf(block_sum(s, red) / C + eps);
+    TOut* o = out + row * os;
+    const float add = one_plus ? 1.f : 0.f;
+    for (int c = threadIdx.x * 8; c < C; c += LN_THREADS * 8) {
+        float v[8], wv[8];
+        load8<TIn>(xr + c, v);
+        load8<float>(w + c, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] * inv * (wv[e] + add);
+        store8<TOut>(o + c, v);
+    }
+}
+
+template <typename TY, typename TC>
+__global__ void __launch_bounds__(LN_THREADS)
+add_rms_norm_vec_kernel(float* __restrict__ stream, const TY* __restrict__ y,
+                        const float* __restrict__ w, int one_plus, float eps,
+                        TC* __restrict__ copy, int C) {
+    __shared__ float red[LN_THREADS / WAVE];
+    const long row = blockIdx.x;
+    const TY* yr = y + row * C;
+    float s = 0.f;
+    for (int c = threadIdx.x * 8; c < C; c += LN_THREADS * 8) {
+        float v[8];
+        load8<TY>(yr + c, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s += v[e] * v[e];
+    }
+    const float inv = 1.f / sqrtf(block_sum(s, red) / C + eps);
+    const float add = one_plus ? 1.f : 0.f;
+    float* xr = stream + row * C;
+    for (int c = threadIdx.x * 8; c < C; c += LN_THREADS * 8) {
+        float v[8], wv[8], xv[8];
+        load8<TY>(yr + c, v);
+        load8<float>(w + c, wv);
+        load8<float>(xr + c, xv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xv[e] += v[e] * inv * (wv[e] + add);
+        store8<float>(xr + c, xv);
+        if (copy) store8<TC>(copy + row * C + c, xv);
+    }
+}
+
 template <typename TIn, typename TOut>
 __global__ void __launch_bounds__(LN_THREADS)
 rms_norm_kernel(const TIn* __restrict__ x, long xs, const float* __restrict__ w, int one_plus,
@@ -1866,8 +1939,13 @@ int nx_rms_norm(const void* x, long xs, int x_bf16, const float* w, int one_plus
                 void* out, long os, int out_bf16, long rows, int C, hipStream_t st) {
     if (rows <= 0) return 0;
     dim3 grid((unsigned)rows), block(LN_THREADS);
-#define RN(TI, TO) rms_norm_kernel<TI, TO><<<grid, block, 0, st>>>( \
-        (const TI*)x, xs, w, one_plus, eps, (TO*)out, os, C)
+    const int xe = x_bf16 ? 2 : 4, oe = out_bf16 ? 2 : 4;
+    const bool vec = (C % 8) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                     ((xs * xe) % 16) == 0 && ((os * oe) % 16) == 0 && ((uintptr_t)w % 16) == 0;
+#define RN(TI, TO) do { if (vec) rms_norm_vec_kernel<TI, TO><<<grid, block, 0, st>>>( \
+        (const TI*)x, xs, w, one_plus, eps, (TO*)out, os, C); \
+    else rms_norm_kernel<TI, TO><<<grid, block, 0, st>>>( \
+        (const TI*)x, xs, w, one_plus, eps, (TO*)out, os, C); } while (0)
     if (x_bf16 && out_bf16) RN(bf16, bf16);
     else if (x_bf16) RN(bf16, float);
     else if (out_bf16) RN(float, bf16);
@@ -1880,6 +1958,15 @@ int nx_add_rms_norm(float* stream, const void* y, int y_bf16, const float* w, in
                     float eps, void* copy_bf16, long rows, int C, hipStream_t st) {
     if (rows <= 0) return 0;
     dim3 grid((unsigned)rows), block(LN_THREADS);
+    const bool vec = (C % 8) == 0 && ((uintptr_t)stream % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
+                     ((uintptr_t)copy_bf16 % 16) == 0 && ((uintptr_t)w % 16) == 0;
+    if (vec) {
+        if (y_bf16) add_rms_norm_vec_kernel<bf16, bf16><<<grid, block, 0, st>>>(
+            stream, (const bf16*)y, w, one_plus, eps, (bf16*)copy_bf16, C);
+        else add_rms_norm_vec_kernel<float, bf16><<<grid, block, 0, st>>>(
+            stream, (const float*)y, w, one_plus, eps, (bf16*)copy_bf16, C);
+        return (int)hipGetLastError();
+    }
     if (y_bf16) add_rms_norm_kernel<bf16, bf16><<<grid, block, 0, st>>>(
         stream, (const bf16*)y, w, one_plus, eps, (bf16*)copy_bf16, C);
     else add_rms_norm_kernel<float, bf16><<<grid, block, 0, st>>>(

@@ -203,21 +203,23 @@ def close(got, want, tol, rtol=0.0):
 # ------------------------------------------------------------ elementwise ops
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("one_plus", [False, True])
-def test_rms_norm_ops(device, one_plus):
+@pytest.mark.parametrize("total,lo,n", [(50, 7, 20), (64, 8, 32)])   # scalar / 16-byte kernels
+def test_rms_norm_ops(device, one_plus, total, lo, n):
     torch.manual_seed(0)
-    wide = torch.randn(2, 5, 50) * 3
-    w = torch.randn(20) * 0.3
-    x = wide[..., 7:27]                                   # a column slice, read in place
+    wide = torch.randn(2, 5, total) * 3
+    w = torch.randn(n) * 0.3
+    x = wide[..., lo:lo + n]                              # a column slice, read in place
     want = oracle.rms(x.double(), EPS) * ((1 + w.double()) if one_plus else w.double())
     got = seqmix.rms_norm(x.to(device), w.to(device), EPS, one_plus, out_dtype=F32)
     close(got.cpu(), want, 1e-5)
-    buf = torch.zeros(2, 5, 33, device=device)            # ... and written into a slice
-    seqmix.rms_norm(x.to(device), w.to(device), EPS, one_plus, out=buf[..., 4:24])
-    close(buf[..., 4:24].cpu(), want, 1e-5)
-    assert float(buf[..., :4].abs().sum() + buf[..., 24:].abs().sum()) == 0.0
+    buf = torch.zeros(2, 5, n + 12, device=device)        # ... and written into a slice
+    seqmix.rms_norm(wide.to(device)[..., lo:lo + n], w.to(device), EPS, one_plus,
+                    out=buf[..., 4:4 + n])
+    close(buf[..., 4:4 + n].cpu(), want, 1e-5)
+    assert float(buf[..., :4].abs().sum() + buf[..., 4 + n:].abs().sum()) == 0.0
     # the post-norm residual step
-    stream = torch.randn(2, 5, 20)
-    y = torch.randn(2, 5, 20) * 4
+    stream = torch.randn(2, 5, n)
+    y = torch.randn(2, 5, n) * 4
     want = stream.double() + oracle.rms(y.double(), EPS) * (
         (1 + w.double()) if one_plus else w.double())
     s = stream.clone().to(device)
@@ -752,6 +754,30 @@ def test_checkpoint_folder_and_schedule_replay(tmp_path):
     close(g0, wa[[0, 7]], 3e-4)
     close(g1, wb[[0]], 3e-4)
     close(g2, torch.stack([wb[8], wa[20]]), 3e-4)
+
+
+def test_command_line_generation(tmp_path, capsys):
+    """inference_demo --model-type soputar: checkpoint folder -> compile ->
+    load -> greedy generation, the same path as every other family."""
+    from safetensors.torch import save_file
+
+    from neuronx_distributed_inference_amd.inference_demo import main
+
+    cfg = model_cfg()
+    W = make_weights(cfg, seed=3)
+    mdir = tmp_path / "model"
+    mdir.mkdir()
+    (mdir / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.bfloat16() for k, v in W.items()}, str(mdir / "model.safetensors"))
+    prompt = tokens_for(cfg, 9, seed=1)
+    rc = main(["--model-type", "soputar", "run", "--model-path", str(mdir),
+               "--compiled-model-path", str(tmp_path / "compiled"),
+               "--prompt-ids", json.dumps([prompt]), "--max-new-tokens", "6",
+               "--torch-dtype", "float32", "--on-cpu", "--seq-len", "32",
+               "--max-context-length", "16"])
+    assert rc == 0
+    printed = [json.loads(l) for l in capsys.readouterr().out.splitlines() if l.startswith("[[")]
+    assert printed and printed[-1][0] == prompt + _oracle_greedy(cfg, W, prompt, 6)
 
 
 def test_config_rejects_what_it_does_not_know():
