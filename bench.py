@@ -144,7 +144,7 @@ def run_hybrid_bench(args):
             # GQA attention, and a layer that borrows the previous one's KV
             mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
             att = {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
-                   "softcap": 20.0, "q_temp": {"coef": 0.5, "every": 64}}
+                   "softcap": 30.0, "q_temp": {"coef": 0.3, "every": 128}}
             quad = [
                 {"type": "latent_attention", "mlp": mlp, "mixer": {
                     "heads": H, "dim": 128, "rot_dim": 64, "vdim": 128,
@@ -163,7 +163,7 @@ def run_hybrid_bench(args):
                 layers.append(lc)
             cfg = SoputarInferenceConfig(
                 neuron_config=ec, architecture="Soputar", width=width, vocab=V,
-                layers=layers, norm={"eps": 1e-5}, embedding={"scale": width ** 0.5})
+                layers=layers, norm={"eps": 1e-5}, embedding={"scale": 8.0})
             cls = SoputarForCausalLM
         else:
             layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff}, "mixer": {

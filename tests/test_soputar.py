@@ -358,18 +358,19 @@ def test_capped_attention_other_shapes(device, L):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("cuts", [None, [300] + [1] * 40])
 def test_capped_attention_far_key_among_hundreds(device, cuts):
-    L = attn_cfg(2, 1, 8, 8, scale=0.6, softcap=50.0, every=64, coef=0.5)
-    _capped_alone(device, L, 340, [(339, 1), (320, 2), (310, 255), (301, 256), (338, 63),
-                                   (337, 64)], page=16, cuts=cuts, tol=5e-5, gain=9.0)
+    L = attn_cfg(2, 1, 8, 8, scale=0.6, softcap=50.0, every=48, coef=0.4)
+    _capped_alone(device, L, 340, [(339, 1), (320, 2), (310, 255), (301, 256), (338, 46),
+                                   (337, 47), (336, 48)], page=16, cuts=cuts, tol=5e-5, gain=9.0)
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("L,cuts", [
     (attn_cfg(4, 2, 32, 64, scale=0.15, softcap=8.0, every=16), None),
-    (attn_cfg(8, 8, 48, 48, scale=0.12, softcap=20.0, every=64), [70, 3, 1, 56]),  # padded tiles
+    (attn_cfg(6, 6, 40, 56, scale=0.12, softcap=15.0, every=32), [70, 3, 1, 56]),  # padded tiles
     (attn_cfg(4, 1, 64, 80, scale=0.1, softcap=0.0, every=0), [2, 64, 64]),
     (attn_cfg(2, 2, 128, 128, scale=0.08), [1, 129]),
     (attn_cfg(4, 2, 40, 24, scale=0.15), None),
+    (attn_cfg(3, 1, 20, 12, scale=0.2), [5, 120, 1, 1, 1, 1, 1]),   # no 16-byte lines: vector kernel
 ])
 def test_capped_attention_bf16_matrix_path_gpu(L, cuts):
     _capped_alone("cuda", L, 130, [(129, 0), (100, 63), (101, 64), (64, 64), (90, 1)],
@@ -474,16 +475,25 @@ def test_latent_attention_far_keys_and_positions(device, cuts):
 @pytest.mark.gpu
 @pytest.mark.parametrize("L,cuts", [
     (latent_cfg(4, 32, 16, 32, 64, scale=0.1), None),
-    (latent_cfg(4, 32, 16, 80, 64, scale=0.1), [3, 60, 1, 66]),      # 80-wide rows
+    (latent_cfg(6, 24, 8, 40, 72, scale=0.1), [3, 60, 1, 66]),       # 80-wide rows, padded
     (latent_cfg(2, 64, 32, 64, 96, scale=0.08, dims=16), [64, 66]),
     # wide rows: 32-key tiles, values split over workgroups, also when decoding
     (latent_cfg(8, 32, 32, 48, 224, scale=0.1), [70, 50] + [1] * 10),
     (latent_cfg(16, 64, 64, 64, 512, scale=0.07), [100] + [1] * 30),
     (latent_cfg(4, 16, 8, 16, 200, scale=0.1), [129, 1]),        # few heads: decode on the vector path
+    (latent_cfg(3, 12, 6, 10, 20, scale=0.2), [100, 29, 1]),     # 26-wide rows: vector kernel
 ])
 def test_latent_attention_bf16_matrix_path_gpu(L, cuts):
     _latent_alone("cuda", L, 130, cuts=cuts, page=16, dtype=BF16, tol=0.03)
     _latent_alone("cuda", L, 130, cuts=[100] + [1] * 30, page=16, dtype=BF16, tol=0.03, fresh=True)
+
+
+@pytest.mark.gpu
+def test_latent_attention_wide_rows_float32_gpu():
+    """32-bit steps never take the matrix-core kernels: 520-wide rows on the
+    vector kernel (its merge area needs more than the default LDS)."""
+    L = latent_cfg(2, 8, 8, 8, 512, scale=0.3)
+    _latent_alone("cuda", L, 40, cuts=[30, 5] + [1] * 5, page=8, tol=1e-4)
 
 
 @pytest.mark.gpu
