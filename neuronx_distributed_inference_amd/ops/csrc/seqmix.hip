@@ -620,6 +620,10 @@ DEV uint16_t f2bf_rne(float f) {
     return (uint16_t)(u >> 16);
 }
 
+// bf16-only kernels take the hardware exponential: its 2^-21 relative error is
+// far below the rounding of their operands
+DEV float fast_tanh_(float y) { return 1.f - __fdividef(2.f, 1.f + __expf(2.f * y)); }
+
 template <int DKP, int DVP, int MA_KT, bool PREFETCH>
 __global__ void __launch_bounds__(256)
 paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __restrict__ kc,
@@ -787,6 +791,10 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         // ---- S^T = K Q^T: lane gets keys 16*kb + 4*lg + r of its own row lr
         float sv[KB][4];
         float mt = -INFINITY;
+        // a tile every row of the workgroup sees whole (all but the diagonal
+        // tiles of a causal prompt) needs no per-score mask
+        const bool whole = nfirst == 0 && base + MA_KT <= n && lo + base + MA_KT - 1 <= i_min &&
+                           i_max - (lo + base) < window;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
             f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -795,6 +803,17 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
                 const bf16x8_t ka = *reinterpret_cast<const bf16x8_t*>(
                     k_lds + (kb * 16 + lr) * KS + ks * 32 + lg * 8);
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[ks], acc, 0, 0, 0);
+            }
+            if (whole && !r1) {                          // uniform
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float x = acc[r] * qscale;
+                    if (cap > 0.f) x = cap * fast_tanh_(x / cap);
+                    if (my_i < 0) x = -INFINITY;
+                    sv[kb][r] = x;
+                    mt = fmaxf(mt, x);
+                }
+                continue;
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -806,7 +825,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
                 if (vis) {
                     x = acc[r] * qscale;
                     if (r1) x -= a1 * __logf(1.f + a2 * (float)dist);
-                    if (cap > 0.f) x = cap * tanhf(x / cap);
+                    if (cap > 0.f) x = cap * fast_tanh_(x / cap);
                 }
                 sv[kb][r] = x;
                 mt = fmaxf(mt, x);
@@ -817,12 +836,12 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         const float m_new = fmaxf(m_run, mt);
         float corr = 1.f, psum = 0.f;
         if (m_new > -INFINITY) {
-            corr = expf(m_run - m_new);
+            corr = __expf(m_run - m_new);
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float pv = sv[kb][r] > -INFINITY ? expf(sv[kb][r] - m_new) : 0.f;
+                    const float pv = sv[kb][r] > -INFINITY ? __expf(sv[kb][r] - m_new) : 0.f;
                     sv[kb][r] = pv;
                     psum += pv;
                 }
@@ -837,23 +856,25 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         l_run = l_run * corr + psum;
         m_run = m_new;
         // ---- rescale O: its rows are 4*lg + r, their corr sits in lane (4*lg + r)
-        float cr[4];
+        if (__any(corr != 1.f)) {                        // some row's maximum moved
+            float cr[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, lg * 4 + r, WAVE);
+            for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, lg * 4 + r, WAVE);
 #pragma unroll
-        for (int nb = 0; nb < DVP / 16; ++nb)
+            for (int nb = 0; nb < DVP / 16; ++nb)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) o_acc[nb][r] *= cr[r];
+                for (int r = 0; r < 4; ++r) o_acc[nb][r] *= cr[r];
+        }
         // ---- O += P V, 32 keys per product, P as hi + lo
 #pragma unroll
         for (int kc2 = 0; kc2 < MA_KT / 32; ++kc2) {
-            union { bf16x8_t v; uint16_t u[8]; } ph, pl;
+            struct { bf16x8_t v; } ph, pl;               // hardware float -> bf16 (RNE)
 #pragma unroll
             for (int jj = 0; jj < 8; ++jj) {
                 const float pv = sv[2 * kc2 + (jj >> 2)][jj & 3];
-                const uint16_t hb = f2bf_rne(pv);
-                ph.u[jj] = hb;
-                pl.u[jj] = f2bf_rne(pv - __uint_as_float((uint32_t)hb << 16));
+                const __bf16 hb = (__bf16)pv;
+                ph.v[jj] = hb;
+                pl.v[jj] = (__bf16)(pv - (float)hb);
             }
 #pragma unroll
             for (int nb = 0; nb < DVP / 16; ++nb) {
@@ -874,8 +895,8 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
     if (sink) {
         const float sk = rsink[myrow];
         const float mf = fmaxf(m_run, sk);
-        const float ca = m_run > -INFINITY ? expf(m_run - mf) : 0.f;
-        fin = ca / (l_run * ca + expf(sk - mf));
+        const float ca = m_run > -INFINITY ? __expf(m_run - mf) : 0.f;
+        fin = ca / (l_run * ca + __expf(sk - mf));
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -1022,11 +1043,11 @@ latent_decode_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float pv = (m_new > -INFINITY && sv[kb][r] > -INFINITY)
-                    ? expf(sv[kb][r] - m_new) : 0.f;
+                    ? __expf(sv[kb][r] - m_new) : 0.f;
                 sv[kb][r] = pv;
                 psum += pv;
             }
-        if (m_new > -INFINITY) corr = expf(m_run - m_new);
+        if (m_new > -INFINITY) corr = __expf(m_run - m_new);
         psum += __shfl_xor(psum, 16, WAVE);
         psum += __shfl_xor(psum, 32, WAVE);
         l_run = l_run * corr + psum;
@@ -1041,13 +1062,13 @@ latent_decode_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* 
         __syncthreads();                                 // V^T complete
         // ---- O += P V for this wave's 128 channels, P as hi + lo
         {
-            union { bf16x8_t v; uint16_t u[8]; } ph, pl;
+            struct { bf16x8_t v; } ph, pl;
 #pragma unroll
             for (int jj = 0; jj < 8; ++jj) {
                 const float pv = sv[jj >> 2][jj & 3];
-                const uint16_t hb = f2bf_rne(pv);
-                ph.u[jj] = hb;
-                pl.u[jj] = f2bf_rne(pv - __uint_as_float((uint32_t)hb << 16));
+                const __bf16 hb = (__bf16)pv;
+                ph.v[jj] = hb;
+                pl.v[jj] = (__bf16)(pv - (float)hb);
             }
 #pragma unroll
             for (int nb = 0; nb < LD_VW / 16; ++nb) {
@@ -1083,8 +1104,8 @@ latent_decode_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* 
     if (sink && hv) {
         const float sk = sink[h];
         const float mf = fmaxf(m_run, sk);
-        const float ca = m_run > -INFINITY ? expf(m_run - mf) : 0.f;
-        fin = ca / (l_run * ca + expf(sk - mf));
+        const float ca = m_run > -INFINITY ? __expf(m_run - mf) : 0.f;
+        fin = ca / (l_run * ca + __expf(sk - mf));
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
