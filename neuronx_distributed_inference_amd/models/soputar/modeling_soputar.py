@@ -65,11 +65,13 @@ class SoputarInferenceConfig(InferenceConfig):
     generic attribute names the engine uses."""
 
     def get_required_attributes(self) -> List[str]:
-        return ["width", "vocab", "layers", "norm", "embedding"]
+        return ["width", "vocab", "layers", "norm"]
 
     def add_derived_config(self):
         if not hasattr(self, "layers"):
             return
+        if not getattr(self, "embedding", None):
+            self.embedding = {"scale": 1.0}       # a file without the entry scales nothing
         self.hidden_size = self.width
         self.vocab_size = self.vocab
         self.num_hidden_layers = len(self.layers)
